@@ -31,7 +31,7 @@ extern "C" {
 
 /* Bumped whenever a signature or a semantic of this header changes; ssd_abi_version() returns the value the library was built
  * with, so a consumer compiled against another header can tell (tests/abi_consumer.c does). */
-#define SSD_HIP_ABI_VERSION 2
+#define SSD_HIP_ABI_VERSION 3
 
 #define SSD_OK 0
 #define SSD_ERR_SHAPE (-1)
@@ -368,6 +368,52 @@ int ssd_allreduce_gr_bf16(const void* in, void* out, long n, int rank, int world
 int ssd_allreduce_add_rmsnorm_gr_bf16(const void* in, const void* res_in, void* res_out, const void* weight, float eps,
                                       void* out_rows, void* out_frag, int T, int H, int rank, int world, void* const* inboxes,
                                       long gr_cap, void* counters, void* err, long spin_budget, void* stream);
+
+/* ---- decoders with an fp32 residual stream, sandwich norms, differential attention and a routed feed-forward (the Fatulix design;
+ * no counterpart in the reference).  `f32` selects the element type of weights, GEMM-input rows and the KV cache: 0 = bf16, 1 = fp32
+ * (true fp32 arithmetic throughout).  Residual rows, norm statistics, attention scores / weights and router logits are fp32 in both. ---- */
+
+/* x_out[t] = table[ids[t]] as fp32 residual rows [T][W]; x0_out (optional) receives the same rows (designs that add the embedding
+ * output again before a repeated pass keep it). */
+int ssd_embed_res32(const int64_t* ids, const void* table_rows, void* x_out, void* x0_out, int T, int W, long vocab, int f32,
+                    void* stream);
+/* out[r] = weight * x[i] / sqrt(mean(x[i]^2) + eps), i = gather[r] or r; x fp32 [.][W].  add (optional, fp32 [T][W], no gather):
+ * x += add first, written back in place. */
+int ssd_rmsnorm_res32(void* x, const void* add, const void* weight, float eps, void* out_rows, const int32_t* gather, int T, int W,
+                      int f32, void* stream);
+/* x += weight * y / sqrt(mean(y^2) + eps): the norm AFTER a sublayer and the residual sum; y fp32 [T][W]. */
+int ssd_rmsnorm_add_res32(const void* y, const void* weight, float eps, void* x, int T, int W, int f32, void* stream);
+/* fp32 rows [rows][ld_src] -> bf16 rows [rows][ld_dst]; columns cols .. ld_dst-1 of dst are set to -inf. */
+int ssd_rows_f32_to_bf16(const void* src, void* dst, int rows, int cols, long ld_src, long ld_dst, void* stream);
+
+/* y = x w^T for row-major x [M][K] and w [N][K] of ANY sizes (csrc/gemm_rows.hip).  epilogue 0: fp32 rows; 1: relu(y)^2 as
+ * element-type rows; 2: element-type rows. */
+int ssd_gemm_rows(const void* x_rows, const void* w_rows, void* y, int M, int N, int K, int epilogue, int f32, void* stream);
+/* The same product per group: sorted rows offsets[e] .. offsets[e+1]-1 (e < E) multiply by w_rows + e * N * K; row_idx (optional)
+ * names the x row of sorted row r as row_idx[r] / idx_div, y rows are the sorted rows.  rows = offsets[E]'s upper bound. */
+int ssd_gemm_rows_grouped(const void* x_rows, const void* w_rows, void* y, const int32_t* offsets, int E, const int32_t* row_idx,
+                          int idx_div, int rows, int N, int K, int epilogue, int f32, void* stream);
+
+/* Differential attention (csrc/attention_diff.hip).  qkvg_rows fp32 [T][H*2*D + G*2*D + G*Dv + H] = [q | k | v | gate logits] with
+ * q and k laid out head by head as [map 1 | map 2]; q_norm_w / k_norm_w [D]; K cache [blocks][G][block_size][2*D], V cache
+ * [blocks][G][block_size][Dv]; slots int32 [T] (-1: no store); q_out [T][H*2*D]; gate_out fp32 [T][H] = sigmoid(gate logits). */
+int ssd_diffattn_store(const void* qkvg_rows, const void* q_norm_w, const void* k_norm_w, float eps, const int32_t* slots,
+                       void* q_out, void* gate_out, void* k_cache, void* v_cache, int T, int H, int G, int D, int Dv, int block_size,
+                       int f32, void* stream);
+/* out[t][h] = out_scale * gate[t][h] * rms_noweight(a_1 - lambda * a_2), a_m = softmax(scale * q_m . k_m) v over keys
+ * 0 .. positions[t] of the token's sequence (cu_q int32 [B+1] row ranges, or q_per_seq rows per sequence when cu_q is NULL). */
+int ssd_diffattn_paged(const void* q_rows, const void* k_cache, const void* v_cache, const void* gate, const int32_t* block_tables,
+                       int max_blocks, const int64_t* positions, const int32_t* cu_q, int q_per_seq, int B, int T, int H, int G,
+                       int D, int Dv, int block_size, float scale, float lambda, float out_scale, float eps, void* out_rows, int f32,
+                       void* stream);
+
+/* Routed feed-forward (csrc/moe.hip): router logits in fp32, the `top` largest per token, softmax over the chosen ones;
+ * counting sort of the (token, slot) pairs by expert; weighted sum of the experts' fp32 output rows (+ the shared expert's). */
+int ssd_moe_route(const void* h_rows, const void* w_router, int32_t* idx, float* weights, int T, int W, int E, int top, int f32,
+                  void* stream);
+int ssd_moe_plan(const int32_t* idx, int T, int top, int E, int32_t* offsets, int32_t* perm, int32_t* inv, void* stream);
+int ssd_moe_combine(const void* y_rows, const int32_t* inv, const float* weights, const void* shared_rows, void* out_rows, int T,
+                    int top, int W, void* stream);
 
 /* hipGraph capture for a host that is not PyTorch -- the reference captures its decode / verify / glue / tree steps with
  * torch.cuda.CUDAGraph (ssd/engine/helpers/cudagraph_helpers.py:20-120); every entry point above only enqueues on `stream`, so the calls

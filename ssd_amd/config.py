@@ -16,6 +16,10 @@ from ssd_amd.model_config import ModelConfig, PRESETS
 
 def resolve_model_config(model: str) -> ModelConfig:
     if os.path.isdir(model):
+        from ssd_amd.model_config import read_native_config
+        native = read_native_config(model)
+        if native is not None:
+            return native
         from transformers import AutoConfig
         return ModelConfig.from_hf(AutoConfig.from_pretrained(model))
     key = model.lower()
@@ -63,6 +67,10 @@ class Config:
     d_model_target: int | None = None
     tokenizer_path: str | None = None
 
+    # arithmetic of the model: "bfloat16" (matrix products and activations in bf16, fp32 accumulation) or "float32" (true fp32
+    # throughout; only model families whose kernels exist in fp32 -- model_runner.MODEL_CLASSES -- accept it)
+    dtype: str = "bfloat16"
+
     verbose: bool = False
     debug_mode: bool = False
     max_steps: int | None = None
@@ -84,6 +92,7 @@ class Config:
 
     def __post_init__(self):
         assert 1 <= self.num_gpus <= 8, "single node only (reference ssd/config.py:55)"
+        assert self.dtype in ("bfloat16", "float32"), self.dtype
         assert self.num_draft_gpus >= 1 and (self.num_draft_gpus == 1 or (self.speculate and self.draft_async)), \
             "num_draft_gpus > 1 needs draft_async"
         if self.hf_config is None:

@@ -1,0 +1,188 @@
+// Row-major GEMM for ANY M, N, K, in bf16 (MFMA 16x16x32, fp32 accumulation) or in true fp32 (FMA), dense or grouped:
+//   y[m][n] = sum_k x[row(m)][k] * w[g(m)][n][k]
+// The skinny / prefill GEMMs of gemm.hip and gemm_pf.hip need fragment-major operands with N % 16 == 0 and K % 32 == 0; models whose
+// sizes do not meet that, grouped (per-expert) products over gathered token rows, and the fp32 arithmetic mode use this kernel.
+// A 256-thread workgroup owns a 64 x 64 output tile; a K step of 32 is staged through LDS with bounds guards (rows or columns past
+// the edge read as zero), so no operand needs padding.  Wave w multiplies token rows 16w..16w+15 by the tile's four 16-feature
+// groups.  Every output element is the sum over k in ascending 32-wide steps, whatever M, the tile or the group is: a row's result does not
+// depend on which other rows share its launch.
+//   grouped: offsets[E+1] cuts the (sorted) rows into E runs, run e multiplies by w + e * N * K; row_idx (optional) names the x row
+//   of every sorted row as row_idx[r] / idx_div; tiles never straddle two runs (blockIdx.y walks a list of at most
+//   ceil(rows / 64) + E tiles, found by a scan of offsets).
+#include "common.h"
+
+namespace {
+
+constexpr int BM = 64, BN = 64, BK = 32;
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+  static __device__ __forceinline__ float ld(const float* p) { return *p; }
+  static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+};
+template <> struct Elem<bf16_t> {
+  static __device__ __forceinline__ float ld(const bf16_t* p) { return bf2f(*p); }
+  static __device__ __forceinline__ void st(bf16_t* p, float v) { *p = (bf16_t)f2bf(v); }
+};
+
+// Stage a [64][32] tile of `src` (row stride ld elements) into LDS (row stride LDT elements); rows >= nrows and columns >= K are zero.
+// 16-byte loads when the row stride and base allow, element loads otherwise.
+template <typename T, int LDT>
+__device__ __forceinline__ void stage_tile(T* lds, const T* __restrict__ src, const int* __restrict__ rowmap, int idx_div, int row0,
+                                           int nrows, int k0, int K, long ld, bool vec_ok) {
+  constexpr int VEC = 16 / sizeof(T);            // elements per 16 bytes
+  constexpr int CPR = BK / VEC;                  // chunks per row
+  for (int c = threadIdx.x; c < 64 * CPR; c += 256) {
+    const int r = c / CPR, kc = (c % CPR) * VEC;
+    const int gr = row0 + r;
+    T tmp[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) tmp[i] = T(0);
+    if (gr < nrows) {
+      const long srow = rowmap ? (long)(rowmap[gr] / idx_div) : (long)gr;
+      const T* p = src + srow * ld + k0 + kc;
+      if (vec_ok && k0 + kc + VEC <= K) {
+        *reinterpret_cast<u32x4_t*>(tmp) = *reinterpret_cast<const u32x4_t*>(p);
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i)
+          if (k0 + kc + i < K) tmp[i] = p[i];
+      }
+    }
+    *reinterpret_cast<u32x4_t*>(lds + r * LDT + kc) = *reinterpret_cast<u32x4_t*>(tmp);
+  }
+}
+
+// epilogue 0: fp32 rows; 1: relu(v)^2 as element-type rows; 2: element-type rows
+template <typename T>
+__device__ __forceinline__ void store_out(void* y, long row, int N, int n, float v, int epi) {
+  if (epi == 0) {
+    reinterpret_cast<float*>(y)[row * N + n] = v;
+  } else {
+    if (epi == 1) { v = v > 0.f ? v : 0.f; v = v * v; }
+    Elem<T>::st(reinterpret_cast<T*>(y) + row * N + n, v);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+gemm_rows_kernel(const T* __restrict__ x, const T* __restrict__ w, void* __restrict__ y, int M, int N, int K, int epi,
+                 const int* __restrict__ offsets, int E, const int* __restrict__ row_idx, int idx_div, bool vec_ok) {
+  constexpr int PAD = 16 / sizeof(T);
+  constexpr int LDT = BK + PAD;
+  __shared__ __attribute__((aligned(16))) T sx[BM * LDT];
+  __shared__ __attribute__((aligned(16))) T sw[BN * LDT];
+  int row0 = blockIdx.y * BM, row_end = M;
+  const T* wg = w;
+  if (offsets) {           // grouped: find the run and the tile inside it that this workgroup owns
+    int tile = blockIdx.y, e = 0;
+    for (; e < E; ++e) {
+      const int cnt = offsets[e + 1] - offsets[e];
+      const int nt = (cnt + BM - 1) / BM;
+      if (tile < nt) break;
+      tile -= nt;
+    }
+    if (e >= E) return;
+    row0 = offsets[e] + tile * BM;
+    row_end = offsets[e + 1];
+    wg = w + (size_t)e * N * K;
+  }
+  const int n0 = blockIdx.x * BN;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+
+  if constexpr (sizeof(T) == 2) {
+    f32x4_t acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < K; k0 += BK) {
+      stage_tile<T, LDT>(sx, x, row_idx, idx_div, row0, row_end, k0, K, K, vec_ok);
+      stage_tile<T, LDT>(sw, wg, nullptr, 1, n0, N, k0, K, K, vec_ok);
+      __syncthreads();
+      const u32x4_t b = *reinterpret_cast<const u32x4_t*>(sx + (wave * 16 + (lane & 15)) * LDT + (lane >> 4) * 8);
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const u32x4_t a = *reinterpret_cast<const u32x4_t*>(sw + (nt * 16 + (lane & 15)) * LDT + (lane >> 4) * 8);
+        acc[nt] = mfma16(a, b, acc[nt]);
+      }
+      __syncthreads();
+    }
+    const int m = row0 + wave * 16 + (lane & 15);
+    if (m < row_end) {
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int n = n0 + nt * 16 + (lane >> 4) * 4 + r;
+          if (n < N) store_out<T>(y, m, N, n, acc[nt][r], epi);
+        }
+    }
+  } else {
+    // fp32: thread (tm, tn) owns token rows tm*4..+3 and features tn*4..+3 of the tile; plain FMA chains in ascending k
+    const int tm = threadIdx.x >> 4, tn = threadIdx.x & 15;
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int k0 = 0; k0 < K; k0 += BK) {
+      stage_tile<T, LDT>(sx, x, row_idx, idx_div, row0, row_end, k0, K, K, vec_ok);
+      stage_tile<T, LDT>(sw, wg, nullptr, 1, n0, N, k0, K, K, vec_ok);
+      __syncthreads();
+#pragma unroll 8
+      for (int k = 0; k < BK; ++k) {
+        float a[4], b[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[i] = (float)sx[(tm * 4 + i) * LDT + k];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b[j] = (float)sw[(tn + 16 * j) * LDT + k];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+      }
+      __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = row0 + tm * 4 + i;
+      if (m >= row_end) continue;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = n0 + tn + 16 * j;
+        if (n < N) store_out<T>(y, m, N, n, acc[i][j], epi);
+      }
+    }
+  }
+}
+
+int launch(const void* x, const void* w, void* y, int M, int N, int K, int epi, const int* offsets, int E, const int* row_idx,
+           int idx_div, int f32, void* stream) {
+  if (!x || !w || !y) return SSD_ERR_ARG;
+  if (M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > 2) return SSD_ERR_SHAPE;
+  if (offsets && E <= 0) return SSD_ERR_SHAPE;
+  const int tiles_m = (M + BM - 1) / BM + (offsets ? E : 0);
+  const dim3 grid((N + BN - 1) / BN, tiles_m);
+  const int esz = f32 ? 4 : 2;
+  const bool vec_ok = ((size_t)K * esz) % 16 == 0 && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
+  if (f32)
+    hipLaunchKernelGGL(gemm_rows_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)x, (const float*)w, y, M, N, K,
+                       epi, offsets, E, row_idx, idx_div < 1 ? 1 : idx_div, vec_ok);
+  else
+    hipLaunchKernelGGL(gemm_rows_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x, (const bf16_t*)w, y, M, N,
+                       K, epi, offsets, E, row_idx, idx_div < 1 ? 1 : idx_div, vec_ok);
+  return hipGetLastError() == hipSuccess ? SSD_OK : SSD_ERR_LAUNCH;
+}
+
+}  // namespace
+
+extern "C" int ssd_gemm_rows(const void* x_rows, const void* w_rows, void* y, int M, int N, int K, int epilogue, int f32,
+                             void* stream) {
+  return launch(x_rows, w_rows, y, M, N, K, epilogue, nullptr, 0, nullptr, 1, f32, stream);
+}
+
+extern "C" int ssd_gemm_rows_grouped(const void* x_rows, const void* w_rows, void* y, const int32_t* offsets, int E,
+                                     const int32_t* row_idx, int idx_div, int rows, int N, int K, int epilogue, int f32,
+                                     void* stream) {
+  if (!offsets) return SSD_ERR_ARG;
+  return launch(x_rows, w_rows, y, rows, N, K, epilogue, offsets, E, row_idx, idx_div, f32, stream);
+}

@@ -26,6 +26,17 @@ from ssd_amd.utils.graphs import capture
 from ssd_amd.engine.async_proto import to_device
 
 
+def model_class(family: str):
+    """The decoder class of a model family (ModelConfig.family / FatulixConfig.family)."""
+    if family == "eagle3":
+        from ssd_amd.eagle import HipEagleDraft
+        return HipEagleDraft
+    if family == "fatulix":
+        from ssd_amd.fatulix import HipFatulix
+        return HipFatulix
+    return HipDecoder
+
+
 class ModelRunner:
     PREFILL_GRAPHS = 4              # prefill shapes kept as hipGraphs
     PREFILL_GRAPH_MAX_T = 1024      # longer prefills are GPU-bound by far: launch overhead does not matter
@@ -55,16 +66,21 @@ class ModelRunner:
         self.max_decode_tokens = max_decode_tokens or dec_tokens
         max_tokens = max(config.max_num_batched_tokens, self.max_decode_tokens)
         eagle = bool(getattr(config, "use_eagle", False))
-        model_cls = HipDecoder
-        if model_cfg.family == "eagle3":
-            from ssd_amd.eagle import HipEagleDraft as model_cls
+        model_cls = model_class(model_cfg.family)
+        dtype = getattr(config, "dtype", "bfloat16")
+        extra = {}
+        if dtype != "bfloat16":
+            if not getattr(model_cls, "supports_float32", False):
+                raise ValueError(f"dtype {dtype!r}: the {model_cfg.family} kernels exist in bfloat16 only")
+            extra["dtype"] = dtype
         # EAGLE-3 target: tap the residual stream entering config.eagle_layers on every forward (reference llama3.py:256-271)
         taps = list(config.eagle_layers) if (eagle and not is_draft) else None
         self.model = model_cls(model_cfg, max_tokens=max_tokens, max_seqs=self.max_bs, max_blocks=self.max_blocks,
                                block_size=self.block_size, max_model_len=config.max_model_len, device=device,
                                tp_rank=tp_rank, tp_size=tp_size, tp_group=tp_group,
                                max_logit_rows=max(self.max_decode_tokens, self.seq_cap),
-                               max_split_tokens=max(256, self.max_decode_tokens), force_collectives=force_collectives, taps=taps)
+                               max_split_tokens=max(256, self.max_decode_tokens), force_collectives=force_collectives, taps=taps,
+                               **extra)
         if weight_source is not None:
             src = weight_source
         elif model_path is not None and W.has_safetensors(model_path) and model_cfg.family == "eagle3":
@@ -498,6 +514,37 @@ class ModelRunner:
         self._log_margins(B, [(s.seq_id, len(s)) for s in seqs])
         toks = self._read_tokens(B)
         return (toks, self.model.full_logits(B)) if draft_return_logits else toks
+
+    @torch.inference_mode()
+    def run_rows(self, seqs, want: list[list[int]]) -> torch.Tensor:
+        """One forward over the not yet cached tokens of `seqs` -- prompt portions of any length beside single decoded tokens, one
+        varlen batch -- that samples nothing: returns the fp32 logits [sum(len(w)), V] of the wanted rows, want[b] = indices among
+        sequence b's new tokens.  The KV of every new token is stored; the caller advances num_cached_tokens."""
+        assert 0 < len(seqs) <= self.seq_cap and len(want) == len(seqs)
+        B = len(seqs)
+        T, max_q = self._prepare_prefill(seqs)
+        self.model.forward(self.d_ids, self.d_pos, T, self._meta("prefill", B, max_q))
+        rows, base = [], 0
+        for s, ws in zip(seqs, want):
+            new = len(s) - (s.num_draft_cached_tokens if self.is_draft else s.num_cached_tokens)
+            assert all(0 <= i < new for i in ws)
+            rows.extend(base + i for i in ws)
+            base += new
+        R = self.model.max_logit_rows
+        if not hasattr(self, "d_rows"):
+            self.d_rows = torch.zeros(R, dtype=torch.int32, device=self.device)
+        out = []
+        for i in range(0, len(rows), R):
+            part = rows[i:i + R]
+            self._upload(self.d_rows, part, torch.int32)
+            n = self.model.compute_logits(T, gather=self.d_rows, rows=len(part))
+            f32 = getattr(self.model, "logits_f32", None)
+            out.append(f32(n).clone() if f32 is not None else self.model.full_logits(n).float())
+            torch.cuda.current_stream().synchronize()       # the pinned staging of d_rows is reused by the next slice
+        torch.cuda.current_stream().synchronize()
+        self._check_collectives()
+        V = self.cfg.vocab_size
+        return torch.cat(out, dim=0) if out else torch.zeros(0, V, dtype=torch.float32, device=self.device)
 
     def eagle_acts(self, n: int) -> torch.Tensor:
         """[n, taps * h] tapped activations of the last prefill / verify forward (reference model_runner.py:613-616); a view

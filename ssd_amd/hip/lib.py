@@ -16,7 +16,7 @@ _LIB = None
 
 c_void_p, c_int, c_long, c_float, c_int64 = C.c_void_p, C.c_int, C.c_long, C.c_float, C.c_int64
 
-ABI_VERSION = 2       # include/ssd_hip.h SSD_HIP_ABI_VERSION (tests/test_abi.py compares the two)
+ABI_VERSION = 3       # include/ssd_hip.h SSD_HIP_ABI_VERSION (tests/test_abi.py compares the two)
 
 # name -> argtypes, exactly include/ssd_hip.h (+ include/ssd_hip_tune.h)
 SIGNATURES = {
@@ -110,6 +110,19 @@ SIGNATURES = {
                          c_void_p, c_int, c_float, c_void_p],
     "ssd_store_step_rows": [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p],
     "ssd_cache_lookup": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p],
+    "ssd_embed_res32": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_void_p],
+    "ssd_rmsnorm_res32": [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ssd_rmsnorm_add_res32": [c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ssd_rows_f32_to_bf16": [c_void_p, c_void_p, c_int, c_int, c_long, c_long, c_void_p],
+    "ssd_gemm_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ssd_gemm_rows_grouped": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ssd_diffattn_store": [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                           c_int, c_int, c_int, c_int, c_void_p],
+    "ssd_diffattn_paged": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                           c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_void_p, c_int, c_void_p],
+    "ssd_moe_route": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ssd_moe_plan": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
+    "ssd_moe_combine": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ssd_draft_advance": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int,
                           c_void_p, c_int, c_void_p],
 }
@@ -119,12 +132,13 @@ def lib_path() -> str:
     return os.path.join(_PKG, "_lib", "libssdhip.so")
 
 
-def build_library(force: bool = False) -> str:
-    """Compile every HIP source for gfx950 (hipcc cross-compiles without a GPU)."""
+def build_library(force: bool = False, quiet: bool = False) -> str:
+    """Compile every HIP source for gfx950 (hipcc cross-compiles without a GPU).  quiet: the build's output goes to stderr."""
     src = os.path.join(_PKG, "csrc")
+    out = dict(stdout=subprocess.DEVNULL) if quiet else {}
     if force:
-        subprocess.check_call(["make", "-C", src, "clean"])
-    subprocess.check_call(["make", "-C", src, "-j8"])
+        subprocess.check_call(["make", "-C", src, "clean"], **out)
+    subprocess.check_call(["make", "-C", src, "-j8"], **out)
     return lib_path()
 
 

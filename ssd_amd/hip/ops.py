@@ -377,3 +377,61 @@ def store_step_rows(src, src_ld: int, dst, B: int, V: int, K: int, step):
     _check(load_library().ssd_store_step_rows(_p(src), src_ld, _p(dst), B, V, K, _p(step), _stream()), "ssd_store_step_rows")
 
 
+
+# ---- fp32-residual decoders: sandwich norms, any-size row-major GEMMs, differential attention, routed feed-forward ----
+
+def embed_res32(ids, table, x_out, x0_out, T: int, W: int, f32: bool):
+    _check(load_library().ssd_embed_res32(_p(ids), _p(table), _p(x_out), _p(x0_out), T, W, table.shape[0], int(f32), _stream()),
+           "ssd_embed_res32")
+
+
+def rmsnorm_res32(x, weight, eps: float, out_rows, T: int, W: int, f32: bool, add=None, gather=None):
+    _check(load_library().ssd_rmsnorm_res32(_p(x), _p(add), _p(weight), eps, _p(out_rows), _p(gather), T, W, int(f32), _stream()),
+           "ssd_rmsnorm_res32")
+
+
+def rmsnorm_add_res32(y, weight, eps: float, x, T: int, W: int, f32: bool):
+    _check(load_library().ssd_rmsnorm_add_res32(_p(y), _p(weight), eps, _p(x), T, W, int(f32), _stream()), "ssd_rmsnorm_add_res32")
+
+
+def rows_f32_to_bf16(src, dst, rows: int, cols: int, ld_src: int, ld_dst: int):
+    _check(load_library().ssd_rows_f32_to_bf16(_p(src), _p(dst), rows, cols, ld_src, ld_dst, _stream()), "ssd_rows_f32_to_bf16")
+
+
+GR_F32, GR_RELU2, GR_ELEM = 0, 1, 2
+
+
+def gemm_rows(x, w, y, M: int, N: int, K: int, f32: bool, epilogue: int = GR_F32):
+    _check(load_library().ssd_gemm_rows(_p(x), _p(w), _p(y), M, N, K, epilogue, int(f32), _stream()), "ssd_gemm_rows")
+
+
+def gemm_rows_grouped(x, w, y, offsets, E: int, rows: int, N: int, K: int, f32: bool, epilogue: int = GR_F32, row_idx=None,
+                      idx_div: int = 1):
+    _check(load_library().ssd_gemm_rows_grouped(_p(x), _p(w), _p(y), _p(offsets), E, _p(row_idx), idx_div, rows, N, K, epilogue,
+                                                int(f32), _stream()), "ssd_gemm_rows_grouped")
+
+
+def diffattn_store(qkvg, q_norm_w, k_norm_w, eps: float, slots, q_out, gate_out, k_cache, v_cache, T, H, G, D, Dv, block_size,
+                   f32: bool):
+    _check(load_library().ssd_diffattn_store(_p(qkvg), _p(q_norm_w), _p(k_norm_w), eps, _p(slots), _p(q_out), _p(gate_out),
+                                             _p(k_cache), _p(v_cache), T, H, G, D, Dv, block_size, int(f32), _stream()),
+           "ssd_diffattn_store")
+
+
+def diffattn_paged(q, k_cache, v_cache, gate, block_tables, max_blocks, positions, B, T, H, G, D, Dv, block_size, scale, lam,
+                   out_scale, eps, out_rows, f32: bool, cu_q=None, q_per_seq: int = 0):
+    _check(load_library().ssd_diffattn_paged(_p(q), _p(k_cache), _p(v_cache), _p(gate), _p(block_tables), max_blocks, _p(positions),
+                                             _p(cu_q), q_per_seq, B, T, H, G, D, Dv, block_size, scale, lam, out_scale, eps,
+                                             _p(out_rows), int(f32), _stream()), "ssd_diffattn_paged")
+
+
+def moe_route(h, w_router, idx, weights, T: int, W: int, E: int, top: int, f32: bool):
+    _check(load_library().ssd_moe_route(_p(h), _p(w_router), _p(idx), _p(weights), T, W, E, top, int(f32), _stream()), "ssd_moe_route")
+
+
+def moe_plan(idx, T: int, top: int, E: int, offsets, perm, inv):
+    _check(load_library().ssd_moe_plan(_p(idx), T, top, E, _p(offsets), _p(perm), _p(inv), _stream()), "ssd_moe_plan")
+
+
+def moe_combine(y, inv, weights, shared, out, T: int, top: int, W: int):
+    _check(load_library().ssd_moe_combine(_p(y), _p(inv), _p(weights), _p(shared), _p(out), T, top, W, _stream()), "ssd_moe_combine")

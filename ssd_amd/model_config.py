@@ -5,7 +5,9 @@ consumes them in ``LlamaAttention`` / ``Qwen3Attention`` (ssd/models/llama3.py:1
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, asdict
+import json
+import os
+from dataclasses import dataclass, asdict, field
 
 
 @dataclass
@@ -97,3 +99,102 @@ PRESETS = {
     "eagle3-llama-3.3-70b": ModelConfig("eagle3", 6144, 1, 48, 8, 128, 16384, 128256, 1e-5, 5e5, 131072, False,
                                         draft_vocab_size=32000, d_model_target=8192),
 }
+
+
+# --------------------------------------------------------------------------------------------------
+# Fatulix: a decoder whose config.json lists its layers one by one (own keys, not a transformers config)
+# --------------------------------------------------------------------------------------------------
+@dataclass
+class RoutedMLP:
+    """Mixture-of-experts feed-forward: `top` of `experts` two-matrix experts (relu^2) per token, plus an optional shared expert."""
+    experts: int
+    top: int
+    ff: int
+    shared_ff: int = 0          # 0: no shared expert
+
+
+@dataclass
+class DiffAttention:
+    """Differential attention: two softmax maps per query head over shared values, per-(head, map) q / k RMS norm, output gate."""
+    heads: int
+    kv_heads: int
+    dim: int                    # query / key size per head and map
+    vdim: int                   # value size per head
+    diff: float                 # the constant of lambda and of the (1 - diff) output scale
+    scale: float                # score scale
+
+
+@dataclass
+class FatulixLayer:
+    mixer: DiffAttention
+    mlp: RoutedMLP | None
+
+
+@dataclass
+class FatulixConfig:
+    """config.json keys: architecture, vocab, width, norm.eps, layers[{type, mixer{heads, kv_heads, dim, vdim, diff, scale},
+    mlp{kind, expert{ff}, router{experts, top}, shared{ff} | null} | null}], loop{start, stop, times}."""
+    vocab_size: int
+    hidden_size: int
+    rms_norm_eps: float
+    layers: list = field(default_factory=list)
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1
+    family: str = "fatulix"
+    max_position_embeddings: int = 1 << 20      # no positional limit: positions do not enter the scores
+    tie_word_embeddings: bool = False
+
+    def runs(self) -> list[tuple[int, int]]:
+        """(layer, pass) of every layer run in execution order.  Layers [loop_start, loop_stop) run loop_times passes with the same
+        weights; every run has KV pages of its own."""
+        a, b = self.loop_start, self.loop_stop
+        span = [(i, ps) for ps in range(self.loop_times) for i in range(a, b)] if b > a else []
+        return [(i, 0) for i in range(a)] + span + [(i, 0) for i in range(max(a, b), len(self.layers))]
+
+    @property
+    def num_layers(self) -> int:            # KV-cache layers = layer runs
+        return len(self.runs())
+
+    def to_dict(self) -> dict:
+        return asdict(self)
+
+    @staticmethod
+    def from_json(cfg: dict) -> "FatulixConfig":
+        layers = []
+        for lc in cfg["layers"]:
+            if lc["type"] != "attention":
+                raise ValueError(f"Fatulix: unknown layer type {lc['type']!r}")
+            m = lc["mixer"]
+            mixer = DiffAttention(int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"]), float(m["diff"]), float(m["scale"]))
+            if mixer.heads % mixer.kv_heads:
+                raise ValueError("Fatulix: heads must be a multiple of kv_heads")
+            ml = lc.get("mlp")
+            mlp = None
+            if ml is not None:
+                if ml.get("kind", "moe") != "moe":
+                    raise ValueError(f"Fatulix: unknown feed-forward kind {ml.get('kind')!r}")
+                sh = ml.get("shared")
+                mlp = RoutedMLP(int(ml["router"]["experts"]), int(ml["router"]["top"]), int(ml["expert"]["ff"]), int(sh["ff"]) if sh else 0)
+            layers.append(FatulixLayer(mixer, mlp))
+        loop = cfg.get("loop") or {}
+        out = FatulixConfig(int(cfg["vocab"]), int(cfg["width"]), float(cfg["norm"]["eps"]), layers, int(loop.get("start", 0)),
+                            int(loop.get("stop", 0)), int(loop.get("times", 1)))
+        if not (0 <= out.loop_start <= max(out.loop_start, out.loop_stop) <= len(layers)) or out.loop_times < 1:
+            raise ValueError("Fatulix: loop out of range")
+        return out
+
+
+# config.json "architecture" values that are read by this package's own readers (everything else goes through transformers' AutoConfig)
+ARCHITECTURES = {"Fatulix": FatulixConfig.from_json}
+
+
+def read_native_config(model_dir: str):
+    """The model configuration of a directory whose config.json names one of ARCHITECTURES, else None."""
+    path = os.path.join(model_dir, "config.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        cfg = json.load(f)
+    reader = ARCHITECTURES.get(cfg.get("architecture")) if isinstance(cfg, dict) else None
+    return reader(cfg) if reader else None

@@ -45,9 +45,35 @@ def eagle_param_shapes(cfg: ModelConfig) -> list[tuple[str, tuple[int, ...]]]:
             ("d2t", (cfg.draft_vocab_size,))]
 
 
+def fatulix_param_shapes(cfg) -> list[tuple[str, tuple[int, ...]]]:
+    """Tensor names and shapes of a Fatulix checkpoint (model_config.FatulixConfig): linear weights [out, in]; layer i's tensors start
+    with 'l<i>.', its mixer's with 'l<i>.mix.', its feed-forward's with 'l<i>.mlp.' (experts 'e<j>', the shared expert 'shared')."""
+    W = cfg.hidden_size
+    out = [("embed", (cfg.vocab_size, W))]
+    for i, lc in enumerate(cfg.layers):
+        p, m = f"l{i}.", lc.mixer
+        out += [(p + "norm1", (W,)), (p + "norm1b", (W,))]
+        if lc.mlp is not None:
+            out += [(p + "norm2", (W,)), (p + "norm2b", (W,))]
+        out += [(p + "mix.q", (m.heads * 2 * m.dim, W)), (p + "mix.k", (m.kv_heads * 2 * m.dim, W)), (p + "mix.v", (m.kv_heads * m.vdim, W)),
+                (p + "mix.q.norm", (m.dim,)), (p + "mix.k.norm", (m.dim,)),
+                (p + "mix.lq1", (m.dim,)), (p + "mix.lk1", (m.dim,)), (p + "mix.lq2", (m.dim,)), (p + "mix.lk2", (m.dim,)),
+                (p + "mix.g", (m.heads, W)), (p + "mix.o", (W, m.heads * m.vdim))]
+        if lc.mlp is not None:
+            for e in range(lc.mlp.experts):
+                out += [(p + f"mlp.e{e}.up", (lc.mlp.ff, W)), (p + f"mlp.e{e}.down", (W, lc.mlp.ff))]
+            out.append((p + "mlp.router", (lc.mlp.experts, W)))
+            if lc.mlp.shared_ff:
+                out += [(p + "mlp.shared.up", (lc.mlp.shared_ff, W)), (p + "mlp.shared.down", (W, lc.mlp.shared_ff))]
+    out += [("final.norm", (W,)), ("head", (cfg.vocab_size, W))]
+    return out
+
+
 def param_shapes(cfg: ModelConfig) -> list[tuple[str, tuple[int, ...]]]:
     if cfg.family == "eagle3":
         return eagle_param_shapes(cfg)
+    if cfg.family == "fatulix":
+        return fatulix_param_shapes(cfg)
     h, hd, nh, nkv, I, V = cfg.hidden_size, cfg.head_dim, cfg.num_heads, cfg.num_kv_heads, cfg.intermediate_size, cfg.vocab_size
     out = [("model.embed_tokens.weight", (V, h))]
     for i in range(cfg.num_layers):
@@ -275,6 +301,7 @@ def synthetic_tensor(name: str, shape, seed: int, std: float, gen_device: str, n
 def shard_param(cfg: ModelConfig, name: str, w: torch.Tensor, rank: int, tp: int) -> torch.Tensor:
     if tp == 1:
         return w
+    assert cfg.family != "fatulix", "Fatulix models are not tensor-parallel"
     hd, nh, nkv, I = cfg.head_dim, cfg.num_heads, cfg.num_kv_heads, cfg.intermediate_size
     if name.endswith("qkv_proj.weight") or name.endswith("qkv_proj.bias"):
         q, k, v = w.split([nh * hd, nkv * hd, nkv * hd], dim=0)

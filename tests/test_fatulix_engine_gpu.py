@@ -1,0 +1,200 @@
+"""The Fatulix decoder through the engine (Config -> ModelRunner -> block manager -> HIP kernels) against the plain whole-sequence
+oracle (oracle/fatulix.py, float64): small self-made configurations with random weights, in fp32 element mode (sharp: any dropped or
+extra key, wrong page, lost pass or stale slot is orders of magnitude above rounding) and in bf16."""
+import json
+import os
+
+import pytest
+import torch
+
+from oracle import fatulix as F
+
+pytestmark = pytest.mark.gpu
+
+
+def write_model(path, cfg, w):
+    from safetensors.torch import save_file
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.contiguous() for k, v in w.items()}, os.path.join(path, "model.safetensors"))
+    return str(path)
+
+
+def row_err(got: torch.Tensor, ref: torch.Tensor) -> torch.Tensor:
+    d = got.double().cpu() - ref.double()
+    d = d - d.mean(-1, keepdim=True)
+    return d.pow(2).mean(-1).sqrt() / ref.double().std()
+
+
+def rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
+    return float(row_err(got, ref).max())
+
+
+def close(got, ref, dtype) -> bool:
+    """fp32: every position within 1e-4 of the logits' spread.  bf16: rounding of the GEMM inputs, and now and then a router decision
+    that bf16 makes the other way at a near-tie: most positions within 4 %, none beyond 25 %."""
+    e = row_err(got, ref)
+    if dtype == "float32":
+        return bool(e.max() < TOL[dtype])
+    return bool(e.median() < 0.04 and e.max() < 0.25)
+
+
+TOL = {"float32": 1e-4, "bfloat16": 6e-2}
+
+# sizes chosen so that nothing the kernels index by coincides: vdim != 2 * dim, heads * vdim != width, per-layer sizes differ
+CONFIGS = {
+    "loop_inside": dict(n_layers=4, loop=(1, 3, 3), no_mlp_layers=(2,), heads=4, kv_heads=2, dim=16, vdim=24, width=64, vocab=96),
+    "mha_top1_noshared": dict(n_layers=2, loop=(0, 0, 1), heads=3, kv_heads=3, dim=20, vdim=12, width=72, vocab=50, experts=3, top=1,
+                              shared_ff=0, ff=40),
+    "mqa_all_experts": dict(n_layers=2, loop=(0, 2, 2), heads=6, kv_heads=1, dim=40, vdim=72, width=100, vocab=131, experts=3, top=3,
+                            ff=24, shared_ff=56, diff=0.45, scale=0.3),
+}
+
+
+def make(name, seed=0):
+    cfg = F.make_config(**CONFIGS[name])
+    if name == "loop_inside":       # layers of one model may differ in every size
+        cfg["layers"][3]["mixer"].update(heads=2, kv_heads=1, dim=24, vdim=40, diff=0.1, scale=0.2)
+        cfg["layers"][3]["mlp"]["router"].update(experts=5, top=3)
+        cfg["layers"][3]["mlp"]["expert"]["ff"] = 16
+    return cfg, F.random_model(cfg, seed)
+
+
+def engine(tmp_path, cfg, w, dtype, max_tokens=512, block_size=16, **kw):
+    from ssd_amd.engine.trace_engine import TraceEngine
+    eng = TraceEngine(write_model(tmp_path / "m", cfg, w), dtype=dtype, max_tokens=max_tokens, block_size=block_size, **kw)
+    for kc, vc in eng.runner.model.kv:          # a slot that is read before it is written shows as NaN
+        kc.fill_(float("nan"))
+        vc.fill_(float("nan"))
+    return eng
+
+
+def tokens(n, vocab, seed):
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_whole_prompt_and_every_layer_run_match_the_oracle(tmp_path, name, dtype):
+    cfg, w = make(name)
+    toks = tokens(83, cfg["vocab"], 1)
+    res = []
+    ref = F.forward(cfg, w, toks, torch.float64, res)
+    eng = engine(tmp_path, cfg, w, dtype)
+    eng.runner.model.tap_residuals = []
+    got = eng.step([{"id": "a", "tokens": toks, "want": list(range(len(toks)))}], ["a"])
+    taps = eng.runner.model.tap_residuals
+    assert len(taps) == len(res) == len(F.layer_runs(cfg))
+    for i, (a, b) in enumerate(zip(taps, res)):
+        assert close(a, b, dtype), f"layer run {i}"
+    assert close(got, ref, dtype)
+
+
+def _replay(eng, rid, toks, cuts, want_all=True):
+    """Feed toks in portions ending at `cuts`; returns the logits of every position."""
+    out, lo = [], 0
+    for hi in cuts:
+        last = hi == len(toks)
+        out.append(eng.step([{"id": rid, "tokens": toks[lo:hi], "want": list(range(hi - lo))}], [rid] if last else []))
+        lo = hi
+    return torch.cat(out)
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_portions_and_token_by_token_decoding_equal_the_whole_prompt(tmp_path, name):
+    cfg, w = make(name, seed=2)
+    n = 70
+    toks = tokens(n, cfg["vocab"], 3)
+    ref = F.forward(cfg, w, toks, torch.float64)
+    eng = engine(tmp_path, cfg, w, "float32", block_size=16)
+    whole = _replay(eng, "w", toks, [n])
+    assert rel_err(whole, ref) < TOL["float32"]
+    schedules = {
+        "token by token": list(range(1, n + 1)),
+        "twos": list(range(2, n + 1, 2)),
+        "page edges": [15, 16, 17, 31, 33, 48, 64, 65, n],
+        "uneven then decode": [3, 10, 11, 40] + list(range(41, n + 1)),
+    }
+    for label, cuts in schedules.items():
+        got = _replay(eng, label, toks, cuts)
+        # a position's arithmetic does not depend on how the prompt was cut: the same sums in the same order
+        assert torch.equal(got, whole), label
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_batches_of_unequal_requests_with_pages_used_again(tmp_path, dtype):
+    cfg, w = make("loop_inside", seed=4)
+    lens = {"a": 50, "b": 7, "c": 33, "d": 1, "e": 45, "f": 20}
+    toks = {k: tokens(n, cfg["vocab"], 10 + i) for i, (k, n) in enumerate(lens.items())}
+    ref = {k: F.forward(cfg, w, t, torch.float64) for k, t in toks.items()}
+    # 8 pages of 16: a + c + e alone need 4 + 3 + 3; the run only fits because ended requests give their pages back
+    eng = engine(tmp_path, cfg, w, dtype, max_tokens=128, block_size=16)
+    got = {k: [] for k in toks}
+    at = {k: 0 for k in toks}
+
+    def step(parts, end=()):
+        entries = []
+        for k, cnt in parts:
+            entries.append({"id": k, "tokens": toks[k][at[k]:at[k] + cnt], "want": list(range(cnt))})
+        lg = eng.step(entries, list(end))
+        r = 0
+        for k, cnt in parts:
+            got[k].append(lg[r:r + cnt])
+            r += cnt
+            at[k] += cnt
+
+    step([("a", 30), ("b", 5), ("d", 1)], end=["d"])
+    step([("a", 1), ("b", 2), ("c", 17)], end=["b"])
+    step([("c", 16), ("a", 19)], end=["a", "c"])          # a and c return 7 pages
+    step([("e", 2), ("f", 19)])
+    step([("f", 1), ("e", 40)], end=["f"])
+    step([("e", 1)])
+    step([("e", 1)])
+    step([("e", 1)], end=["e"])
+    assert not eng.live and len(eng.blocks.free_block_ids) == 8
+    for k in toks:
+        assert close(torch.cat(got[k]), ref[k], dtype), (k, rel_err(torch.cat(got[k]), ref[k]))
+
+
+def test_long_decoding_over_many_pages(tmp_path):
+    cfg, w = make("mqa_all_experts", seed=5)
+    n = 230
+    toks = tokens(n, cfg["vocab"], 6)
+    ref = F.forward(cfg, w, toks, torch.float64)
+    eng = engine(tmp_path, cfg, w, "float32", max_tokens=256, block_size=16)
+    got = _replay(eng, "x", toks, [3] + list(range(4, n + 1)))
+    assert rel_err(got, ref) < TOL["float32"]
+
+
+def test_pool_and_live_limits_are_enforced(tmp_path):
+    cfg, w = make("mha_top1_noshared")
+    eng = engine(tmp_path, cfg, w, "bfloat16", max_tokens=64, block_size=16, max_live=2)
+    eng.step([{"id": "a", "tokens": tokens(40, cfg["vocab"], 0), "want": []}])
+    with pytest.raises(RuntimeError):
+        eng.step([{"id": "b", "tokens": tokens(30, cfg["vocab"], 1), "want": []}])       # 3 + 2 pages > 4
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_llm_generate(tmp_path, dtype):
+    """The framework's own entry point and scheduler: batched prefill, batched decode (hipGraph replays), paged KV, argmax kernels."""
+    from ssd_amd import LLM, SamplingParams
+    cfg, w = make("loop_inside", seed=7)
+    path = write_model(tmp_path / "m", cfg, w)
+    prompts = [tokens(n, cfg["vocab"], 20 + n) for n in (5, 19, 1, 34)]
+    new = 24
+    llm = LLM(path, dtype=dtype, kvcache_block_size=16, num_kvcache_blocks=32, max_num_seqs=3, max_model_len=128,
+              max_num_batched_tokens=128)
+    outs, _ = llm.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=new, ignore_eos=True), use_tqdm=False)
+    assert len(outs) == len(prompts)
+    for p, o in zip(prompts, outs):
+        gen = o["token_ids"]
+        assert len(gen) == new
+        # teacher forcing: every generated token is the oracle's argmax of its step, or within rounding of it
+        lg = F.forward(cfg, w, p + gen[:-1], torch.float64)[len(p) - 1:]
+        top = lg.max(-1).values
+        chosen = lg[torch.arange(new), torch.tensor(gen)]
+        margin = 1e-3 if dtype == "float32" else 0.15
+        assert ((top - chosen) <= margin * lg.std()).all(), (top - chosen).max()
+        if dtype == "float32":
+            assert gen == lg.argmax(-1).tolist()

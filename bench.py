@@ -69,7 +69,10 @@ def parse(argv=None):
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=40)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c4", choices=["c4", "c3", "c2", "c5t", "c4e", "tiny", "tiny-async", "tiny-eagle"])
+    ap.add_argument("--workload", default="c4", choices=["c4", "c3", "c2", "c5t", "c4e", "tiny", "tiny-async", "tiny-eagle", "fatulix"])
+    ap.add_argument("--arch-size", default="all", help="--workload fatulix: one of the sizes in ssd_amd/utils/arch_bench.py SIZES, or all")
+    ap.add_argument("--arch-batch", type=int, default=0, help="--workload fatulix: decode batch (0 = 1 and 8)")
+    ap.add_argument("--arch-only", default="both", choices=["both", "fatulix", "llama"], help="--workload fatulix: which family to run")
     ap.add_argument("--k", type=int, default=None, help="speculation length (default: 7 async, 6 sync)")
     ap.add_argument("--f", type=int, default=3, help="async fan-out")
     ap.add_argument("--placement", default="auto", choices=["auto", "colocated", "dedicated"])
@@ -429,6 +432,10 @@ def cpu_baseline():
 
 def main():
     args = parse()
+    if args.workload == "fatulix":      # the Fatulix decoder beside an equal-size Llama decoder (ssd_amd/utils/arch_bench.py); single GPU
+        from ssd_amd.utils.arch_bench import run as arch_run
+        print(json.dumps(arch_run(args)), flush=True)
+        return
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         sys.exit(self_launch(args))
     world = int(os.environ.get("WORLD_SIZE", "1"))

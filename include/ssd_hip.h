@@ -396,16 +396,18 @@ int ssd_gemm_rows_grouped(const void* x_rows, const void* w_rows, void* y, const
 
 /* Differential attention (csrc/attention_diff.hip).  qkvg_rows fp32 [T][H*2*D + G*2*D + G*Dv + H] = [q | k | v | gate logits] with
  * q and k laid out head by head as [map 1 | map 2]; q_norm_w / k_norm_w [D]; K cache [blocks][G][block_size][2*D], V cache
- * [blocks][G][block_size][Dv]; slots int32 [T] (-1: no store); q_out [T][H*2*D]; gate_out fp32 [T][H] = sigmoid(gate logits). */
+ * transposed per page [blocks][G][Dv][block_size]; slots int32 [T] (-1: no store); q_out [T][H*2*D]; gate_out fp32 [T][H] = sigmoid(gate logits). */
 int ssd_diffattn_store(const void* qkvg_rows, const void* q_norm_w, const void* k_norm_w, float eps, const int32_t* slots,
                        void* q_out, void* gate_out, void* k_cache, void* v_cache, int T, int H, int G, int D, int Dv, int block_size,
                        int f32, void* stream);
 /* out[t][h] = out_scale * gate[t][h] * rms_noweight(a_1 - lambda * a_2), a_m = softmax(scale * q_m . k_m) v over keys
- * 0 .. positions[t] of the token's sequence (cu_q int32 [B+1] row ranges, or q_per_seq rows per sequence when cu_q is NULL). */
+ * 0 .. positions[t] of the token's sequence (cu_q int32 [B+1] row ranges, or q_per_seq rows per sequence when cu_q is NULL).
+ * context_lens int32 [B] (keys each sequence holds) and max_q (most rows of one sequence) are optional (NULL / 0); with them, bf16,
+ * D % 8 == 0, D <= 128, Dv % 16 == 0, Dv <= 128 and block_size % 32 == 0 the MFMA form runs, else the fp32 scalar form. */
 int ssd_diffattn_paged(const void* q_rows, const void* k_cache, const void* v_cache, const void* gate, const int32_t* block_tables,
-                       int max_blocks, const int64_t* positions, const int32_t* cu_q, int q_per_seq, int B, int T, int H, int G,
-                       int D, int Dv, int block_size, float scale, float lambda, float out_scale, float eps, void* out_rows, int f32,
-                       void* stream);
+                       int max_blocks, const int64_t* positions, const int32_t* context_lens, const int32_t* cu_q, int q_per_seq,
+                       int max_q, int B, int T, int H, int G, int D, int Dv, int block_size, float scale, float lambda, float out_scale,
+                       float eps, void* out_rows, int f32, void* stream);
 
 /* Routed feed-forward (csrc/moe.hip): router logits in fp32, the `top` largest per token, softmax over the chosen ones;
  * counting sort of the (token, slot) pairs by expert; weighted sum of the experts' fp32 output rows (+ the shared expert's). */

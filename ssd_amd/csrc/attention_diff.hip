@@ -2,7 +2,8 @@
 //     o = rms_noweight(a_1 - lambda * a_2) * out_scale * gate,      a_m = softmax(scale * q_m . k_m) v,
 // with per-(head, map) RMS norm of q and k (weight shared by all heads and maps), no rotation, and a per-head sigmoid gate.
 // Query / key size D and value size Dv are independent and arbitrary (any D, Dv <= 512); element type bf16 or fp32 (`f32`).
-//   cache layout per layer: K [blocks][G][block_size][2 * D] (map 1 | map 2, normalised), V [blocks][G][block_size][Dv].
+//   cache layout per layer: K [blocks][G][block_size][2 * D] (map 1 | map 2, normalised), V TRANSPOSED per page [blocks][G][Dv][block_size]
+//   (the keys of a page are contiguous per value column: the weighted sum's MFMA operand is a plain 8-byte load).
 //   * ssd_diffattn_store   from the fused projection's fp32 rows [q | k | v | gate logits]: norm q -> q_out, norm k -> K cache at
 //                          slots[t], v -> V cache, sigmoid(gate logits) -> gate_out fp32 [T][H].  slot -1: nothing is stored.
 //   * ssd_diffattn_paged   one workgroup per (token, head): its 4 waves take 64-key tiles round-robin; inside a tile a lane owns
@@ -57,7 +58,7 @@ diffattn_store_kernel(const float* __restrict__ qkvg, const T* __restrict__ qw, 
   if (slot >= 0) {
     for (int c = threadIdx.x; c < Nv; c += 256) {
       const int g = c / Dv, d = c % Dv;
-      stf<T>(vc + (((size_t)blk * G + g) * bs + off) * Dv + d, row[Nq + Nk + c]);
+      stf<T>(vc + (((size_t)blk * G + g) * Dv + d) * bs + off, row[Nq + Nk + c]);
     }
   }
   for (int h = threadIdx.x; h < H; h += 256) gate_out[(size_t)t * H + h] = 1.0f / (1.0f + expf(-row[Nq + Nk + Nv + h]));
@@ -75,7 +76,7 @@ diffattn_paged_kernel(const T* __restrict__ q, const T* __restrict__ kc, const T
   // ---- LDS carve-up ----
   float* sq = smem;                          // [2 * D] the two query vectors
   float* sp = sq + 2 * D;                    // [4 waves][2 maps][64] weights of the current tile
-  long* srow = reinterpret_cast<long*>(sp + 4 * 2 * 64);   // [4 waves][64] cache row of every key of the tile (8-byte aligned: 2D + 512 floats)
+  long* srow = reinterpret_cast<long*>(sp + 4 * 2 * 64);   // [4 waves][64] V^T address of every key of the tile (8-byte aligned: 2D + 512 floats)
   float* sacc = reinterpret_cast<float*>(srow + 4 * 64);    // [4 waves][2 maps][Dv] partial sums
   float* sml = sacc + 4 * 2 * Dv;            // [4 waves][4] m1, l1, m2, l2
   float* sred = sml + 16;                    // [4]
@@ -109,8 +110,9 @@ diffattn_paged_kernel(const T* __restrict__ q, const T* __restrict__ kc, const T
     float s1 = -INFINITY, s2 = -INFINITY;
     long crow = 0;
     if (j < nkeys) {
-      crow = ((long)table[j / bs] * G + g) * bs + (j % bs);
-      const T* kr = kc + (size_t)crow * 2 * D;
+      const long pg = (long)table[j / bs] * G + g;
+      crow = pg * Dv * bs + (j % bs);                  // element (value 0, this key) of the page's transposed V
+      const T* kr = kc + (size_t)(pg * bs + (j % bs)) * 2 * D;
       float d1 = 0.f, d2 = 0.f;
       for (int d = 0; d < D; ++d) {
         d1 = fmaf(sq[d], ldf<T>(kr + d), d1);
@@ -133,11 +135,11 @@ diffattn_paged_kernel(const T* __restrict__ q, const T* __restrict__ kc, const T
     for (int i = 0; i < DA_MAXV; ++i) { a1[i] *= c1; a2[i] *= c2; }
     for (int jj = 0; jj < cnt; ++jj) {
       const float w1 = p1[jj], w2 = p2[jj];
-      const T* vr = vc + (size_t)rowp[jj] * Dv;
+      const T* vr = vc + (size_t)rowp[jj];
 #pragma unroll
       for (int i = 0; i < DA_MAXV; ++i) {
         const int d = lane + i * 64;
-        if (d < Dv) { const float v = ldf<T>(vr + d); a1[i] = fmaf(w1, v, a1[i]); a2[i] = fmaf(w2, v, a2[i]); }
+        if (d < Dv) { const float v = ldf<T>(vr + (size_t)d * bs); a1[i] = fmaf(w1, v, a1[i]); a2[i] = fmaf(w2, v, a2[i]); }
       }
     }
     __builtin_amdgcn_wave_barrier();
@@ -184,6 +186,226 @@ diffattn_paged_kernel(const T* __restrict__ q, const T* __restrict__ kc, const T
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// MFMA form (bf16, D % 8 == 0, D <= 128, Dv % 16 == 0, Dv <= 128, block_size % 32 == 0).  For one kv head, the query ROWS of a
+// sequence are its (token, head of the group) pairs; a wave owns 16 rows and walks the keys in steps of 32 (never across a page):
+//   S_m[key][row]  = K_m tile (A operand, loaded from the cache rows as they lie) x Q_m (B operand, in registers)   -- 16x16x32, fp32
+//   online softmax per row and map in fp32 on the accumulator fragments (a lane holds 8 keys of one row)
+//   O_m[dv][row]  += V^T tile (A operand: 2 x 8-byte loads from the transposed page) x P_m (B operand: the lane's 8 weights, bf16)
+// The k slots of the second product are the keys in the order the first product's fragments hold them, so no data moves between lanes.
+// tile mode  (prompt portions): workgroup = 4 waves = 64 consecutive rows of one sequence, every wave scans keys 0 .. its last row's position.
+// split mode (<= 16 rows per sequence: decoding): the 4 waves share the rows and split the keys; partial (max, sum, O) merge in LDS
+//            in wave order.
+// Keys past a row's position are masked by select (whatever the cache holds there); V of keys past the sequence's length is zeroed.
+// ---------------------------------------------------------------------------------------------------------------------
+constexpr int DM_KS = 4, DM_DVT = 8;
+
+__device__ __forceinline__ float quad_max(float v) { v = fmaxf(v, __shfl_xor(v, 16, 64)); return fmaxf(v, __shfl_xor(v, 32, 64)); }
+__device__ __forceinline__ float quad_sum(float v) { v += __shfl_xor(v, 16, 64); return v + __shfl_xor(v, 32, 64); }
+
+__global__ void __launch_bounds__(256)
+diffattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vt,
+                     const float* __restrict__ gate, const int32_t* __restrict__ bt, int max_blocks,
+                     const int64_t* __restrict__ positions, const int32_t* __restrict__ ctx_lens, const int32_t* __restrict__ cu_q,
+                     int q_per_seq, int B, int H, int G, int D, int Dv, int bs, float scale, float lambda, float out_scale, float eps,
+                     bf16_t* __restrict__ out, int split) {
+  extern __shared__ float smem[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, qd = lane >> 4;
+  const int g = blockIdx.y, R = H / G;
+  const int KS = (D + 31) >> 5, DVT = Dv >> 4;
+  // ---- which sequence, which rows ----
+  int b = 0, tile = blockIdx.x, tok0 = 0, qb = 0;
+  if (split) {
+    b = blockIdx.x; tile = 0;
+    tok0 = cu_q ? cu_q[b] : b * q_per_seq;
+    qb = cu_q ? cu_q[b + 1] - cu_q[b] : q_per_seq;
+  } else {
+    for (; b < B; ++b) {
+      tok0 = cu_q ? cu_q[b] : b * q_per_seq;
+      qb = cu_q ? cu_q[b + 1] - cu_q[b] : q_per_seq;
+      const int nt = (qb * R + 63) >> 6;
+      if (tile < nt) break;
+      tile -= nt;
+    }
+    if (b >= B) return;
+  }
+  const int nrows = qb * R;
+  const int row0 = split ? 0 : tile * 64 + wave * 16;
+  if (!split && row0 >= nrows) return;                 // (tile mode has no workgroup barriers)
+  const int row = row0 + r;
+  const bool valid = row < nrows;
+  const int rr = valid ? row : row0;
+  const int token = tok0 + rr / R, head = g * R + rr % R;
+  const int pos = (int)positions[token];
+  const int ctx = ctx_lens[b];
+  int maxpos = pos;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) maxpos = max(maxpos, __shfl_xor(maxpos, o, 64));
+  const int32_t* table = bt + (size_t)b * max_blocks;
+
+  // ---- Q in registers: B operand, lane (row r, dims ks*32 + qd*8 ..+7) ----
+  u32x4_t qreg[2][DM_KS];
+  const bf16_t* qrow = q + ((size_t)token * H + head) * 2 * D;
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int ks = 0; ks < DM_KS; ++ks) {
+      qreg[m][ks] = u32x4_t{0u, 0u, 0u, 0u};
+      const int d0 = ks * 32 + qd * 8;
+      if (ks < KS && d0 < D && valid) qreg[m][ks] = *reinterpret_cast<const u32x4_t*>(qrow + m * D + d0);
+    }
+
+  float mx[2] = {-INFINITY, -INFINITY}, ls[2] = {0.f, 0.f};
+  f32x4_t acc[2][DM_DVT];
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int i = 0; i < DM_DVT; ++i) acc[m][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const int nsteps = (maxpos >> 5) + 1;
+  int s_begin = 0, s_end = nsteps;
+  if (split) { const int per = (nsteps + 3) >> 2; s_begin = wave * per; s_end = min(nsteps, s_begin + per); }
+
+  for (int st = s_begin; st < s_end; ++st) {
+    const int k0 = st << 5;
+    const size_t pg = (size_t)table[k0 / bs] * G + g;
+    const int koff = k0 % bs;
+    f32x4_t s[2][2];
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+      for (int hg = 0; hg < 2; ++hg) {
+        s[m][hg] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        const bf16_t* kr = kc + (pg * bs + koff + hg * 16 + r) * 2 * D + m * D + qd * 8;
+#pragma unroll
+        for (int ks = 0; ks < DM_KS; ++ks) {
+          if (ks < KS) {
+            u32x4_t a = {0u, 0u, 0u, 0u};
+            if (ks * 32 + qd * 8 < D) a = *reinterpret_cast<const u32x4_t*>(kr + ks * 32);
+            s[m][hg] = mfma16(a, qreg[m][ks], s[m][hg]);
+          }
+        }
+      }
+    u32x4_t pb[2];
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      float v[8];
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int hg = 0; hg < 2; ++hg)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int key = k0 + hg * 16 + qd * 4 + e;
+          const float x = key <= pos ? s[m][hg][e] * scale : -INFINITY;
+          v[hg * 4 + e] = x;
+          tmax = fmaxf(tmax, x);
+        }
+      tmax = quad_max(tmax);
+      const float mnew = fmaxf(mx[m], tmax);
+      const float msafe = mnew == -INFINITY ? 0.f : mnew;
+      const float corr = __expf(mx[m] - msafe);
+      float psum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { v[e] = __expf(v[e] - msafe); psum += v[e]; }
+      psum = quad_sum(psum);
+      ls[m] = ls[m] * corr + psum;
+      mx[m] = mnew;
+#pragma unroll
+      for (int i = 0; i < DM_DVT; ++i) acc[m][i] *= corr;
+      pb[m] = u32x4_t{pack_bf2(v[0], v[1]), pack_bf2(v[2], v[3]), pack_bf2(v[4], v[5]), pack_bf2(v[6], v[7])};
+    }
+    const bool tail = k0 + 32 > ctx;
+#pragma unroll
+    for (int i = 0; i < DM_DVT; ++i) {
+      if (i < DVT) {
+        const bf16_t* vp = vt + (pg * Dv + i * 16 + r) * bs + koff + qd * 4;
+        u32x2_t lo = *reinterpret_cast<const u32x2_t*>(vp);
+        u32x2_t hi = *reinterpret_cast<const u32x2_t*>(vp + 16);
+        if (tail) {         // keys past the sequence: whatever the page holds there must not meet a zero weight as NaN
+          const int kb = k0 + qd * 4;
+          if (kb + 0 >= ctx) lo.x &= 0xffff0000u;
+          if (kb + 1 >= ctx) lo.x &= 0x0000ffffu;
+          if (kb + 2 >= ctx) lo.y &= 0xffff0000u;
+          if (kb + 3 >= ctx) lo.y &= 0x0000ffffu;
+          if (kb + 16 >= ctx) hi.x &= 0xffff0000u;
+          if (kb + 17 >= ctx) hi.x &= 0x0000ffffu;
+          if (kb + 18 >= ctx) hi.y &= 0xffff0000u;
+          if (kb + 19 >= ctx) hi.y &= 0x0000ffffu;
+        }
+        const u32x4_t a = {lo.x, lo.y, hi.x, hi.y};
+        acc[0][i] = mfma16(a, pb[0], acc[0][i]);
+        acc[1][i] = mfma16(a, pb[1], acc[1][i]);
+      }
+    }
+  }
+
+  if (split) {
+    // ---- merge the four waves' partials in wave order ----
+    float* sm = smem;                       // [4 waves][2 maps][2: max, sum][16 rows]
+    float* sbuf = smem + 4 * 2 * 2 * 16;    // [2 maps][DVT][64 lanes][4]
+    if (qd == 0) {
+#pragma unroll
+      for (int m = 0; m < 2; ++m) { sm[((wave * 2 + m) * 2 + 0) * 16 + r] = mx[m]; sm[((wave * 2 + m) * 2 + 1) * 16 + r] = ls[m]; }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      float M = -INFINITY;
+      for (int w = 0; w < 4; ++w) M = fmaxf(M, sm[((w * 2 + m) * 2 + 0) * 16 + r]);
+      float L = 0.f;
+      for (int w = 0; w < 4; ++w) {
+        const float mw = sm[((w * 2 + m) * 2 + 0) * 16 + r];
+        L += mw == -INFINITY ? 0.f : sm[((w * 2 + m) * 2 + 1) * 16 + r] * __expf(mw - M);
+      }
+      const float f = mx[m] == -INFINITY ? 0.f : __expf(mx[m] - M);
+#pragma unroll
+      for (int i = 0; i < DM_DVT; ++i) acc[m][i] *= f;
+      ls[m] = L;
+    }
+    for (int w = 1; w < 4; ++w) {
+      if (wave == w) {
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+          for (int i = 0; i < DM_DVT; ++i)
+            if (i < DVT) *reinterpret_cast<f32x4_t*>(sbuf + ((size_t)(m * DVT + i) * 64 + lane) * 4) = acc[m][i];
+      }
+      __syncthreads();
+      if (wave == 0) {
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+          for (int i = 0; i < DM_DVT; ++i)
+            if (i < DVT) acc[m][i] += *reinterpret_cast<const f32x4_t*>(sbuf + ((size_t)(m * DVT + i) * 64 + lane) * 4);
+      }
+      __syncthreads();
+    }
+    if (wave != 0) return;
+  }
+
+  // ---- combine the maps, norm over the head's values, scale, gate; lane (row r, values i*16 + qd*4 ..+3) ----
+  const float i1 = 1.0f / ls[0], i2 = lambda / ls[1];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < DM_DVT; ++i)
+    if (i < DVT) {
+      acc[0][i] = acc[0][i] * i1 - acc[1][i] * i2;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += acc[0][i][e] * acc[0][i][e];
+    }
+  ss = quad_sum(ss);
+  const float rn = out_scale * gate[(size_t)token * H + head] / sqrtf(ss / (float)Dv + eps);
+  if (valid) {
+    bf16_t* orow = out + ((size_t)token * H + head) * Dv + qd * 4;
+#pragma unroll
+    for (int i = 0; i < DM_DVT; ++i)
+      if (i < DVT) {
+        const u32x2_t o = {pack_bf2(acc[0][i][0] * rn, acc[0][i][1] * rn), pack_bf2(acc[0][i][2] * rn, acc[0][i][3] * rn)};
+        *reinterpret_cast<u32x2_t*>(orow + i * 16) = o;
+      }
+  }
+}
+
 }  // namespace
 
 #define LAUNCH_OK() (hipGetLastError() == hipSuccess ? SSD_OK : SSD_ERR_LAUNCH)
@@ -205,13 +427,25 @@ extern "C" int ssd_diffattn_store(const void* qkvg_rows, const void* q_norm_w, c
 }
 
 extern "C" int ssd_diffattn_paged(const void* q_rows, const void* k_cache, const void* v_cache, const void* gate,
-                                  const int32_t* block_tables, int max_blocks, const int64_t* positions, const int32_t* cu_q,
-                                  int q_per_seq, int B, int T, int H, int G, int D, int Dv, int block_size, float scale, float lambda,
-                                  float out_scale, float eps, void* out_rows, int f32, void* stream) {
+                                  const int32_t* block_tables, int max_blocks, const int64_t* positions, const int32_t* context_lens,
+                                  const int32_t* cu_q, int q_per_seq, int max_q, int B, int T, int H, int G, int D, int Dv,
+                                  int block_size, float scale, float lambda, float out_scale, float eps, void* out_rows, int f32,
+                                  void* stream) {
   if (!q_rows || !k_cache || !v_cache || !gate || !block_tables || !positions || !out_rows) return SSD_ERR_ARG;
   if (T <= 0 || B <= 0 || H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || Dv > 64 * DA_MAXV || block_size <= 0 || max_blocks <= 0)
     return SSD_ERR_SHAPE;
   if (!cu_q && q_per_seq <= 0) return SSD_ERR_ARG;
+  if (!f32 && context_lens && max_q > 0 && D % 8 == 0 && D <= 32 * DM_KS && Dv % 16 == 0 && Dv <= 16 * DM_DVT && block_size % 32 == 0 &&
+      (2 * D * 2) % 16 == 0) {
+    const int R = H / G;
+    const int split = max_q * R <= 16 ? 1 : 0;
+    const int gx = split ? B : ((long)T * R + 63) / 64 + B;
+    const size_t lds_m = split ? (size_t)(4 * 2 * 2 * 16 + 2 * (Dv / 16) * 64 * 4) * 4 : 0;
+    hipLaunchKernelGGL(diffattn_mfma_kernel, dim3(gx, G), dim3(256), lds_m, (hipStream_t)stream, (const bf16_t*)q_rows,
+                       (const bf16_t*)k_cache, (const bf16_t*)v_cache, (const float*)gate, block_tables, max_blocks, positions,
+                       context_lens, cu_q, q_per_seq, B, H, G, D, Dv, block_size, scale, lambda, out_scale, eps, (bf16_t*)out_rows, split);
+    return LAUNCH_OK();
+  }
   const size_t lds = (size_t)(2 * D + 4 * 2 * 64) * 4 + 4 * 64 * 8 + (size_t)(4 * 2 * Dv + 16 + 4) * 4 + 8;
   if (lds > 64 * 1024) return SSD_ERR_SHAPE;
   if (f32)

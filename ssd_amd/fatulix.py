@@ -143,13 +143,13 @@ class HipFatulix:
                    for li, _ in self.runs)
 
     def alloc_kv(self, num_blocks: int) -> None:
-        """Per layer run: K [blocks][G][block_size][2 * dim] (both maps, normalised), V [blocks][G][block_size][vdim]."""
+        """Per layer run: K [blocks][G][block_size][2 * dim] (both maps, normalised), V transposed per page [blocks][G][vdim][block_size]."""
         self.num_blocks = num_blocks
         self.kv = []
         for li, _ in self.runs:
             m = self.cfg.layers[li].mixer
             self.kv.append((torch.zeros(num_blocks, m.kv_heads, self.block_size, 2 * m.dim, dtype=self.elem, device=self.device),
-                            torch.zeros(num_blocks, m.kv_heads, self.block_size, m.vdim, dtype=self.elem, device=self.device)))
+                            torch.zeros(num_blocks, m.kv_heads, m.vdim, self.block_size, dtype=self.elem, device=self.device)))
 
     # ---------------------------------------------------------------------------------------------
     def launch_mixer(self, run: int, li: int, T: int, positions, meta: AttnMeta) -> None:
@@ -162,7 +162,7 @@ class HipFatulix:
                          T, m.heads, m.kv_heads, m.dim, m.vdim, self.block_size, f)
         H.diffattn_paged(self.q, kc, vc, self.gate, meta.block_tables, self.max_blocks, positions, meta.B, T, m.heads, m.kv_heads,
                          m.dim, m.vdim, self.block_size, m.scale, self.lam[li], 1.0 - m.diff, cfg.rms_norm_eps, self.att, f,
-                         cu_q=meta.cu_q, q_per_seq=meta.q_per_seq)
+                         cu_q=meta.cu_q, q_per_seq=meta.q_per_seq, context_lens=meta.context_lens, max_q=meta.max_q)
         H.gemm_rows(self.att, w[p + "o"], self.y, T, self.W, m.heads * m.vdim, f)
 
     def launch_mlp(self, li: int, T: int) -> None:

@@ -419,10 +419,11 @@ def diffattn_store(qkvg, q_norm_w, k_norm_w, eps: float, slots, q_out, gate_out,
 
 
 def diffattn_paged(q, k_cache, v_cache, gate, block_tables, max_blocks, positions, B, T, H, G, D, Dv, block_size, scale, lam,
-                   out_scale, eps, out_rows, f32: bool, cu_q=None, q_per_seq: int = 0):
+                   out_scale, eps, out_rows, f32: bool, cu_q=None, q_per_seq: int = 0, context_lens=None, max_q: int = 0):
+    """context_lens + max_q given (and bf16, aligned head sizes, block_size % 32 == 0): the MFMA form; else the scalar fp32 form."""
     _check(load_library().ssd_diffattn_paged(_p(q), _p(k_cache), _p(v_cache), _p(gate), _p(block_tables), max_blocks, _p(positions),
-                                             _p(cu_q), q_per_seq, B, T, H, G, D, Dv, block_size, scale, lam, out_scale, eps,
-                                             _p(out_rows), int(f32), _stream()), "ssd_diffattn_paged")
+                                             _p(context_lens), _p(cu_q), q_per_seq, max_q, B, T, H, G, D, Dv, block_size, scale, lam,
+                                             out_scale, eps, _p(out_rows), int(f32), _stream()), "ssd_diffattn_paged")
 
 
 def moe_route(h, w_router, idx, weights, T: int, W: int, E: int, top: int, f32: bool):

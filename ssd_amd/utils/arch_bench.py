@@ -1,0 +1,128 @@
+"""bench.py --workload fatulix: prefill and decode throughput of the Fatulix decoder at layer sizes that resemble real models (random
+weights), beside the closest existing family -- a dense grouped-query Llama decoder -- at equal active size: the same width, query /
+key / value / output projection sizes (two 64-wide maps per head = one 128-wide head), the same feed-forward parameters per token
+(top * 2 * ff + 2 * shared_ff = 3 * intermediate), layers, vocabulary, prompt and batch.  Both run through the same ModelRunner paths
+(`run(seqs, is_prefill)`: staging, varlen prefill / hipGraph decode, LM head, argmax)."""
+from __future__ import annotations
+
+import json
+import time
+
+import torch
+
+from ssd_amd.config import Config
+from ssd_amd.engine.block_manager import BlockManager
+from ssd_amd.engine.sequence import Sequence
+from ssd_amd.model_config import DiffAttention, FatulixConfig, FatulixLayer, ModelConfig, RoutedMLP
+
+VOCAB = 32000
+SIZES = {
+    # name: (width, layers, heads, kv heads, experts, top, expert ff, shared ff, dense intermediate of the equal Llama)
+    "w2048": (2048, 4, 16, 4, 8, 2, 1536, 3072, 4096),
+    "w4096": (4096, 4, 32, 8, 16, 2, 3072, 6144, 8192),
+}
+
+
+def models(size: str):
+    W, L, Hh, G, E, top, ff, sff, inter = SIZES[size]
+    assert top * 2 * ff + 2 * sff == 3 * inter
+    layer = FatulixLayer(DiffAttention(Hh, G, 64, 128, 0.25, 64 ** -0.5), RoutedMLP(E, top, ff, sff))
+    fat = FatulixConfig(VOCAB, W, 1e-5, [layer] * L)
+    llama = ModelConfig("llama", W, L, Hh, G, 128, inter, VOCAB, 1e-5, 5e5, 131072, False)
+    return fat, llama
+
+
+def _runner(cfg, max_len: int, batch: int, dtype: str = "bfloat16"):
+    from ssd_amd.engine.model_runner import ModelRunner
+    bs = 256
+    blocks = batch * (-(-max_len // bs)) + 2
+    config = Config("synthetic", hf_config=cfg, dtype=dtype, kvcache_block_size=bs, max_num_seqs=batch, max_model_len=max_len,
+                    max_num_batched_tokens=max(max_len, 4096), num_kvcache_blocks=blocks)
+    Sequence.block_size = bs
+    runner = ModelRunner(config, cfg, is_draft=False, device=torch.device("cuda", 0), weights_seed=0, num_kvcache_blocks=blocks)
+    return runner, BlockManager(blocks, bs, max_model_len=max_len, prefix_cache=False)
+
+
+def _timed(fn, steps: int, warmup: int) -> float:
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def measure(cfg, prompt_len: int, batch: int, steps: int, warmup: int) -> dict:
+    """Prefill of ONE prompt_len-token prompt (eager, as the engine prefills) and `batch` sequences decoding from that context."""
+    max_len = prompt_len + steps + warmup + 8
+    runner, bm = _runner(cfg, max_len, batch)
+    g = torch.Generator().manual_seed(0)
+    prompts = [torch.randint(0, cfg.vocab_size, (prompt_len,), generator=g).tolist() for _ in range(batch)]
+
+    def prefill_once():
+        s = Sequence(prompts[0])
+        bm.allocate(s)
+        runner.run([s], True)
+        bm.deallocate(s)
+
+    t_pf = _timed(prefill_once, max(3, steps // 8), 2)
+    seqs = []
+    for p in prompts:
+        s = Sequence(p)
+        bm.allocate(s)
+        tok = runner.run([s], True)[0]
+        s.append_token(tok)
+        s.num_cached_tokens = len(s) - 1
+        seqs.append(s)
+
+    def decode_once():
+        for s in seqs:
+            bm.may_append(s, 1)
+        toks = runner.run(seqs, False)
+        for s, t in zip(seqs, toks):
+            s.append_token(t)
+            s.num_cached_tokens = len(s) - 1
+
+    t_dec = _timed(decode_once, steps, warmup)
+    out = {"prefill_tok_s": round(prompt_len / t_pf, 1), "prefill_ms": round(t_pf * 1e3, 3), "decode_tok_s": round(batch / t_dec, 1),
+           "decode_ms_per_step": round(t_dec * 1e3, 3)}
+    m = runner.model
+    if hasattr(m, "active_weight_bytes"):
+        out["decode_weight_gb"] = round(m.active_weight_bytes(batch) / 1e9, 3)
+    else:
+        out["decode_weight_gb"] = round(m.weight_bytes() / 1e9, 3)
+    out["decode_hbm_roofline_frac"] = round(out["decode_weight_gb"] * 1e9 / t_dec / 8e12, 3)
+    runner.exit()
+    del runner
+    torch.cuda.empty_cache()
+    return out
+
+
+def run(args) -> dict:
+    steps, warmup = args.steps, args.warmup
+    prompt_len = args.input_len if args.input_len != 128 else 2048
+    results = {}
+    sizes = list(SIZES) if getattr(args, "arch_size", "all") == "all" else [args.arch_size]
+    batches = (1, 8) if not getattr(args, "arch_batch", 0) else (args.arch_batch,)
+    only = getattr(args, "arch_only", "both")
+    for size in sizes:
+        fat, llama = models(size)
+        for batch in batches:
+            key = f"{size} prompt={prompt_len} batch={batch}"
+            results[key] = {}
+            if only in ("both", "fatulix"):
+                results[key]["fatulix"] = measure(fat, prompt_len, batch, steps, warmup)
+            if only in ("both", "llama"):
+                results[key]["llama_equal_size"] = measure(llama, prompt_len, batch, steps, warmup)
+            print(f"[arch_bench] {key}: {json.dumps(results[key])}", flush=True)
+    k = f"w4096 prompt={prompt_len} batch=8"
+    if k not in results or len(results[k]) < 2:
+        return {"metric": "Fatulix / equal-size Llama throughput (partial run)", "sizes": results}
+    return {"metric": "decode tokens/s, Fatulix w4096 (4 layers, 16 experts top 2 + shared), batch 8, beside an equal-size Llama decoder",
+            "value": results[k]["fatulix"]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": results[k]["fatulix"]["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic (random weights, random tokens)",
+            "config": {"model": "fatulix-w4096-synthetic", "global_batch": 8, "seq_len": prompt_len, "parallelism": "single GPU"},
+            "closest_model_value": results[k]["llama_equal_size"]["decode_tok_s"], "sizes": results}

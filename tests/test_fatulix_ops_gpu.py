@@ -131,23 +131,31 @@ def test_route_plan_combine(f32, E, top):
     torch.testing.assert_close(out.double(), ref, rtol=1e-5, atol=1e-5)
 
 
-def _diffattn_ref(q, k, v, gate, scale, lam, out_scale, eps):
-    """q [T][H][2][D], k [T][G][2][D], v [T][G][Dv] (one sequence, causal), float64."""
-    T, Hh, _, D = q.shape
-    G = k.shape[1]
-    mask = torch.ones(T, T, dtype=torch.bool, device=q.device).tril()
-    out = []
-    for h in range(Hh):
-        kv = h // (Hh // G)
-        a = [torch.softmax(((q[:, h, m] @ k[:, kv, m].T) * scale).masked_fill(~mask, float("-inf")), -1) @ v[:, kv] for m in range(2)]
-        o = a[0] - lam * a[1]
-        o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * out_scale * gate[:, h:h + 1]
-        out.append(o)
-    return torch.cat(out, -1)
+def _paged_ref(qo, kc, vt, gate, bt, pos, seq, Hh, G, D, Dv, bs, scale, lam, osc, eps):
+    """Token by token from what the CACHE holds (K [blk][G][bs][2D], V^T [blk][G][Dv][bs]): float64, keys 0 .. pos[t] of sequence seq[t]."""
+    T = qo.shape[0]
+    q = qo.double().view(T, Hh, 2, D)
+    out = torch.zeros(T, Hh * Dv, dtype=torch.float64, device=qo.device)
+    for t in range(T):
+        n = int(pos[t]) + 1
+        j = torch.arange(n, device=qo.device)
+        pg = bt[int(seq[t])].long()[j // bs]
+        K = kc[pg, :, j % bs].double().view(n, G, 2, D)
+        V = vt[pg, :, :, j % bs].double()                       # [n][G][Dv]
+        for h in range(Hh):
+            g = h // (Hh // G)
+            a = [torch.softmax((K[:, g, m] @ q[t, h, m]) * scale, 0) @ V[:, g] for m in range(2)]
+            o = a[0] - lam * a[1]
+            out[t, h * Dv:(h + 1) * Dv] = o / torch.sqrt((o * o).mean() + eps) * osc * gate[t, h].double()
+    return out
+
+
+SHAPES = [(4, 2, 56, 80, 64), (8, 2, 64, 128, 32), (4, 4, 128, 64, 64), (5, 5, 8, 16, 32),          # the MFMA form takes these in bf16
+          (3, 3, 20, 24, 16), (6, 1, 64, 40, 32), (2, 2, 136, 512 - 8, 64)]                          # scalar form only
 
 
 @pytest.mark.parametrize("f32", MODES)
-@pytest.mark.parametrize("Hh,G,D,Dv,bs", [(4, 2, 56, 80, 64), (3, 3, 20, 24, 16), (6, 1, 64, 40, 32), (2, 2, 136, 520 - 8, 64)])
+@pytest.mark.parametrize("Hh,G,D,Dv,bs", SHAPES)
 def test_diffattn_store_and_paged_over_scattered_pages(f32, Hh, G, D, Dv, bs):
     from ssd_amd.hip import ops as H
     g = torch.Generator().manual_seed(D + Dv)
@@ -163,8 +171,8 @@ def test_diffattn_store_and_paged_over_scattered_pages(f32, Hh, G, D, Dv, bs):
     bt = bt.to(DEV)
     pos = torch.arange(T, dtype=torch.int64, device=DEV)
     slots = torch.tensor([pages[p // bs] * bs + p % bs for p in range(T)], dtype=torch.int32, device=DEV)
-    kc = torch.zeros(nblk, G, bs, 2 * D, dtype=el, device=DEV)
-    vc = torch.zeros(nblk, G, bs, Dv, dtype=el, device=DEV)
+    kc = torch.full((nblk, G, bs, 2 * D), float("nan"), dtype=el, device=DEV)
+    vc = torch.full((nblk, G, Dv, bs), float("nan"), dtype=el, device=DEV)
     qo = torch.zeros(T, Hh * 2 * D, dtype=el, device=DEV)
     gate = torch.zeros(T, Hh, device=DEV)
     H.diffattn_store(qkvg, qw, kw, eps, slots, qo, gate, kc, vc, T, Hh, G, D, Dv, bs, f32)
@@ -178,11 +186,68 @@ def test_diffattn_store_and_paged_over_scattered_pages(f32, Hh, G, D, Dv, bs):
     torch.testing.assert_close(gate.double(), torch.sigmoid(x[:, nq + nk + nv:]), rtol=1e-5, atol=1e-6)
     blk, off = (slots // bs).long(), (slots % bs).long()
     torch.testing.assert_close(kc[blk, :, off].double().view(T, G, 2, D), k_ref, **_tol(f32))
-    torch.testing.assert_close(vc[blk, :, off].double(), v_ref, **_tol(f32))
-    out = torch.zeros(T, Hh * Dv, dtype=el, device=DEV)
+    torch.testing.assert_close(vc[blk, :, :, off].double(), v_ref, **_tol(f32))
+    # keys that stand out, far back and at page borders: map 1 of head 0 looks at key 0 from every later position, map 2 at the last
+    # key of the first page; a key that is skipped or mixed up is an O(1) error
+    qn = qo.double().view(T, Hh, 2, D)
+    kc[pages[0], 0, 0, :D] = (6 * qn[T - 1, 0, 0] / qn[T - 1, 0, 0].norm() * D ** 0.5).to(el)
+    kc[pages[0], 0, bs - 1, D:] = (6 * qn[T - 1, 0, 1] / qn[T - 1, 0, 1].norm() * D ** 0.5).to(el)
+    seq = torch.zeros(T, dtype=torch.int64)
+    ref = _paged_ref(qo, kc, vc, gate, bt, pos, seq, Hh, G, D, Dv, bs, scale, lam, osc, eps)
+    tol = dict(rtol=1e-4, atol=1e-4) if f32 else dict(rtol=2e-2, atol=2e-2)
     cu = torch.tensor([0, T], dtype=torch.int32, device=DEV)
-    H.diffattn_paged(qo, kc, vc, gate, bt, nblk, pos, 1, T, Hh, G, D, Dv, bs, scale, lam, osc, eps, out, f32, cu_q=cu)
-    # the reference attends over what the cache holds (the stored roundings), so only the attention arithmetic is compared
-    ref = _diffattn_ref(qo.double().view(T, Hh, 2, D), kc[blk, :, off].double().view(T, G, 2, D), vc[blk, :, off].double(), gate.double(),
-                        scale, lam, osc, eps)
-    torch.testing.assert_close(out.double(), ref, **(dict(rtol=1e-4, atol=1e-4) if f32 else dict(rtol=1.6e-2, atol=1.6e-2)))
+    ctx = torch.tensor([T], dtype=torch.int32, device=DEV)
+    for fast in (False, True):          # the scalar form, then (where the shape allows it in bf16) the MFMA form
+        out = torch.zeros(T, Hh * Dv, dtype=el, device=DEV)
+        H.diffattn_paged(qo, kc, vc, gate, bt, nblk, pos, 1, T, Hh, G, D, Dv, bs, scale, lam, osc, eps, out, f32, cu_q=cu,
+                         **(dict(context_lens=ctx, max_q=T) if fast else {}))
+        torch.testing.assert_close(out.double(), ref, **tol)
+
+
+@pytest.mark.parametrize("f32", MODES)
+@pytest.mark.parametrize("Hh,G,D,Dv,bs", SHAPES[:5])
+def test_diffattn_decode_rows_of_several_sequences(f32, Hh, G, D, Dv, bs):
+    """A batch of sequences with different lengths bringing one or two rows each (decoding, the last tokens of a portion): keys just
+    inside the visible range count, the key after a row's position does not (the second row's key is in the cache when the first row
+    attends), page borders fall at and next to the positions, unwritten slots hold NaN."""
+    from ssd_amd.hip import ops as H
+    g = torch.Generator().manual_seed(Hh * 100 + D)
+    eps, scale, lam, osc = 1e-6, 0.3, 0.45, 0.9
+    el = _elem(f32)
+    lens = [bs + 1, 2 * bs, 1, 3 * bs - 1, 2]             # context lengths INCLUDING the new rows
+    new = [1, 2, 1, 2, 2]
+    B, nblk = len(lens), 16
+    order = torch.randperm(nblk, generator=g).tolist()
+    bt = torch.full((B, nblk), -1, dtype=torch.int32)
+    tables, at = [], 0
+    for b, n in enumerate(lens):
+        k = -(-n // bs)
+        tables.append(order[at:at + k]); at += k
+        bt[b, :k] = torch.tensor(tables[-1], dtype=torch.int32)
+    bt = bt.to(DEV)
+    kc = torch.full((nblk, G, bs, 2 * D), float("nan"), dtype=el, device=DEV)
+    vc = torch.full((nblk, G, Dv, bs), float("nan"), dtype=el, device=DEV)
+    N = Hh * 2 * D + G * 2 * D + G * Dv + Hh
+    qw, kw = _rand((D,), f32, g) + 1, _rand((D,), f32, g) + 1
+    # fill every sequence's context through the store kernel, then the rows of this step are its last `new` tokens
+    rows_q, rows_gate, pos, seq = [], [], [], []
+    for b, n in enumerate(lens):
+        x = (torch.randn(n, N, generator=g) * 1.5).to(DEV)
+        slots = torch.tensor([tables[b][p // bs] * bs + p % bs for p in range(n)], dtype=torch.int32, device=DEV)
+        qo = torch.zeros(n, Hh * 2 * D, dtype=el, device=DEV)
+        gt = torch.zeros(n, Hh, device=DEV)
+        H.diffattn_store(x, qw, kw, eps, slots, qo, gt, kc, vc, n, Hh, G, D, Dv, bs, f32)
+        rows_q.append(qo[n - new[b]:]); rows_gate.append(gt[n - new[b]:])
+        pos += list(range(n - new[b], n)); seq += [b] * new[b]
+    q, gate = torch.cat(rows_q).contiguous(), torch.cat(rows_gate).contiguous()
+    T = q.shape[0]
+    posd = torch.tensor(pos, dtype=torch.int64, device=DEV)
+    cu = torch.tensor([0] + torch.tensor(new).cumsum(0).tolist(), dtype=torch.int32, device=DEV)
+    ctx = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    ref = _paged_ref(q, kc, vc, gate, bt, posd, torch.tensor(seq), Hh, G, D, Dv, bs, scale, lam, osc, eps)
+    tol = dict(rtol=1e-4, atol=1e-4) if f32 else dict(rtol=2e-2, atol=2e-2)
+    for fast in (False, True):
+        out = torch.zeros(T, Hh * Dv, dtype=el, device=DEV)
+        H.diffattn_paged(q, kc, vc, gate, bt, nblk, posd, B, T, Hh, G, D, Dv, bs, scale, lam, osc, eps, out, f32, cu_q=cu,
+                         **(dict(context_lens=ctx, max_q=2) if fast else {}))
+        torch.testing.assert_close(out.double(), ref, **tol)

@@ -409,10 +409,10 @@ int ssd_diffattn_paged(const void* q_rows, const void* k_cache, const void* v_ca
                        int max_q, int B, int T, int H, int G, int D, int Dv, int block_size, float scale, float lambda, float out_scale,
                        float eps, void* out_rows, int f32, void* stream);
 
-/* Routed feed-forward (csrc/moe.hip): router logits in fp32, the `top` largest per token, softmax over the chosen ones;
+/* Routed feed-forward (csrc/moe.hip): from the router's fp32 logits [T][E] (ssd_gemm_rows, fp32 rows out) the `top` largest per token,
+ * softmax over the chosen ones;
  * counting sort of the (token, slot) pairs by expert; weighted sum of the experts' fp32 output rows (+ the shared expert's). */
-int ssd_moe_route(const void* h_rows, const void* w_router, int32_t* idx, float* weights, int T, int W, int E, int top, int f32,
-                  void* stream);
+int ssd_moe_route(const float* logits, int32_t* idx, float* weights, int T, int E, int top, void* stream);
 int ssd_moe_plan(const int32_t* idx, int T, int top, int E, int32_t* offsets, int32_t* perm, int32_t* inv, void* stream);
 int ssd_moe_combine(const void* y_rows, const int32_t* inv, const float* weights, const void* shared_rows, void* out_rows, int T,
                     int top, int W, void* stream);

@@ -2,7 +2,7 @@
 //   y[m][n] = sum_k x[row(m)][k] * w[g(m)][n][k]
 // The skinny / prefill GEMMs of gemm.hip and gemm_pf.hip need fragment-major operands with N % 16 == 0 and K % 32 == 0; models whose
 // sizes do not meet that, grouped (per-expert) products over gathered token rows, and the fp32 arithmetic mode use this kernel.
-// A 256-thread workgroup owns a 64 x 64 output tile; a K step of 32 is staged through LDS with bounds guards (rows or columns past
+// Few token rows in bf16 take the skinny weight-streaming form below; otherwise a 256-thread workgroup owns a 64 x 64 output tile; a K step of 32 is staged through LDS with bounds guards (rows or columns past
 // the edge read as zero), so no operand needs padding.  Wave w multiplies token rows 16w..16w+15 by the tile's four 16-feature
 // groups.  Every output element is the sum over k in ascending 32-wide steps, whatever M, the tile or the group is: a row's result does not
 // depend on which other rows share its launch.
@@ -155,11 +155,96 @@ gemm_rows_kernel(const T* __restrict__ x, const T* __restrict__ w, void* __restr
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// Skinny form (bf16, K % 8 == 0, few token rows: decoding): a weight-streaming product.  A workgroup owns 16 features; its NW waves take
+// the 32-wide k-tiles round-robin in runs of U, so the workgroup as a whole walks its 16 weight rows linearly; both MFMA operands are
+// 16-byte loads straight from the row-major matrices (lane = (row & 15) + 16 * (k chunk)); the waves' partial tiles are summed through
+// LDS in wave order.  Grouped: blockIdx.y is the group; a group with no rows exits at once, one with more than 16 rows loops over
+// 16-row chunks.
+// ---------------------------------------------------------------------------------------------------------------------
+template <int NW>
+__global__ void __launch_bounds__(NW * 64)
+gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ y, int M, int N, int K, int epi,
+                   const int* __restrict__ offsets, const int* __restrict__ row_idx, int idx_div) {
+  constexpr int U = 4;
+  __shared__ f32x4_t red[NW * 64];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, qd = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  int m_begin = 0, m_end = M;
+  const bf16_t* wg = w;
+  if (offsets) {
+    m_begin = offsets[blockIdx.y];
+    m_end = offsets[blockIdx.y + 1];
+    if (m_begin >= m_end) return;
+    wg = w + (size_t)blockIdx.y * N * K;
+  }
+  const int nrow = min(n0 + r, N - 1);
+  const bf16_t* wp = wg + (size_t)nrow * K + qd * 8;
+  const int KT = (K + 31) >> 5;
+  for (int m0 = m_begin; m0 < m_end; m0 += 16) {
+    const int mrow = m0 + r;
+    const bool mvalid = mrow < m_end;
+    const long xrow = mvalid ? (row_idx ? (long)(row_idx[mrow] / idx_div) : (long)mrow) : 0;
+    const bf16_t* xp = x + xrow * K + qd * 8;
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (int kt0 = wave * U; kt0 < KT; kt0 += NW * U) {
+      u32x4_t a[U], b[U];
+#pragma unroll
+      for (int i = 0; i < U; ++i) {
+        const int kt = kt0 + i;
+        const bool ok = kt < KT && kt * 32 + qd * 8 < K;
+        a[i] = u32x4_t{0u, 0u, 0u, 0u};
+        b[i] = u32x4_t{0u, 0u, 0u, 0u};
+        if (ok) a[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wp + kt * 32));
+        if (ok && mvalid) b[i] = *reinterpret_cast<const u32x4_t*>(xp + kt * 32);
+      }
+#pragma unroll
+      for (int i = 0; i < U; ++i) acc = mfma16(a[i], b[i], acc);
+    }
+    red[wave * 64 + lane] = acc;
+    __syncthreads();
+    if (wave == 0) {
+      f32x4_t sum = red[lane];
+#pragma unroll
+      for (int wv = 1; wv < NW; ++wv) sum += red[wv * 64 + lane];
+      if (mvalid) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int n = n0 + qd * 4 + e;
+          if (n < N) store_out<bf16_t>(y, mrow, N, n, sum[e], epi);
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+constexpr int SKINNY_MAX_ROWS = 16, SKINNY_MAX_GROUPED_ROWS = 64;
+
 int launch(const void* x, const void* w, void* y, int M, int N, int K, int epi, const int* offsets, int E, const int* row_idx,
            int idx_div, int f32, void* stream) {
   if (!x || !w || !y) return SSD_ERR_ARG;
   if (M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > 2) return SSD_ERR_SHAPE;
   if (offsets && E <= 0) return SSD_ERR_SHAPE;
+  if (!f32 && K % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 &&
+      M <= (offsets ? SKINNY_MAX_GROUPED_ROWS : SKINNY_MAX_ROWS)) {
+    const int groups = (N + 15) / 16;
+    const dim3 sg(groups, offsets ? E : 1);
+    const int id = idx_div < 1 ? 1 : idx_div;
+    const long wgs = (long)groups * (offsets ? (M < E ? M : E) : 1);          // workgroups that have rows
+    // few workgroups: more waves each (a CU pulls from HBM what its waves have in flight), as long as every wave gets k-tiles
+    const int kt = (K + 31) / 32;
+    if (wgs < 256 && kt >= 64)
+      hipLaunchKernelGGL(gemm_skinny_kernel<16>, sg, dim3(1024), 0, (hipStream_t)stream, (const bf16_t*)x, (const bf16_t*)w, y, M, N, K,
+                         epi, offsets, row_idx, id);
+    else if (wgs < 1024 && kt >= 32)
+      hipLaunchKernelGGL(gemm_skinny_kernel<8>, sg, dim3(512), 0, (hipStream_t)stream, (const bf16_t*)x, (const bf16_t*)w, y, M, N, K,
+                         epi, offsets, row_idx, id);
+    else
+      hipLaunchKernelGGL(gemm_skinny_kernel<4>, sg, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x, (const bf16_t*)w, y, M, N, K,
+                         epi, offsets, row_idx, id);
+    return hipGetLastError() == hipSuccess ? SSD_OK : SSD_ERR_LAUNCH;
+  }
   const int tiles_m = (M + BM - 1) / BM + (offsets ? E : 0);
   const dim3 grid((N + BN - 1) / BN, tiles_m);
   const int esz = f32 ? 4 : 2;

@@ -1,5 +1,6 @@
 // Routed feed-forward (mixture of experts) around the grouped GEMM of gemm_rows.hip:
-//   ssd_moe_route    z = W_r h in fp32; the `top` largest logits per token (lowest index wins a tie) and the softmax over them
+//   ssd_moe_route    from the router's fp32 logits z = W_r h (a GEMM with fp32 rows out): the `top` largest per token (lowest index
+//                    wins a tie) and the softmax over them
 //   ssd_moe_plan     counting sort of the T * top (token, slot) pairs by expert: offsets[E+1], perm (sorted row -> pair), inv (pair -> sorted row)
 //   ssd_moe_combine  out[t] = sum_j weight[t][j] * y[inv[t * top + j]] (+ shared[t]) in slot order, fp32
 // Between plan and combine the caller runs the experts as two grouped GEMMs over the sorted rows (up with the activation as epilogue,
@@ -9,44 +10,32 @@
 
 namespace {
 
-template <typename T> __device__ __forceinline__ float ldf(const T* p);
-template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
-template <> __device__ __forceinline__ float ldf<bf16_t>(const bf16_t* p) { return bf2f(*p); }
-
 constexpr int MOE_MAX_E = 4096, MOE_MAX_TOP = 32;
 
-template <typename T>
-__global__ void __launch_bounds__(256)
-moe_route_kernel(const T* __restrict__ h, const T* __restrict__ wr, int32_t* __restrict__ idx, float* __restrict__ wt, int W, int E,
-                 int top) {
+__global__ void __launch_bounds__(64)
+moe_route_kernel(const float* __restrict__ zin, int32_t* __restrict__ idx, float* __restrict__ wt, int E, int top) {
   extern __shared__ float z[];      // [E]
-  const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const T* hr = h + (size_t)t * W;
-  for (int e = wave; e < E; e += 4) {
-    const T* wrow = wr + (size_t)e * W;
-    float s = 0.f;
-    for (int k = lane; k < W; k += 64) s = fmaf(ldf<T>(hr + k), ldf<T>(wrow + k), s);
-    s = wave_sum(s);
-    if (lane == 0) z[e] = s;
-  }
+  const int t = blockIdx.x, lane = threadIdx.x;
+  for (int e = lane; e < E; e += 64) z[e] = zin[(size_t)t * E + e];
   __syncthreads();
-  if (threadIdx.x == 0) {
-    float val[MOE_MAX_TOP];
-    for (int j = 0; j < top; ++j) {
-      float best = -INFINITY; int bi = 0;
-      for (int e = 0; e < E; ++e) {
-        const float v = z[e];
-        if (v > best) { best = v; bi = e; }
-      }
-      val[j] = best;
-      idx[(size_t)t * top + j] = bi;
-      z[bi] = -INFINITY;
+  // `top` rounds of a wave-wide argmax; among equal logits the lowest index wins
+  float vmax = 0.f, den = 0.f, myval = 0.f;
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY; int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) { const float v = z[e]; if (v > best) { best = v; bi = e; } }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(best, o, 64); const int oi = __shfl_xor(bi, o, 64);
+      if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
     }
-    float den = 0.f;
-    const float vmax = val[0];
-    for (int j = 0; j < top; ++j) { val[j] = expf(val[j] - vmax); den += val[j]; }
-    for (int j = 0; j < top; ++j) wt[(size_t)t * top + j] = val[j] / den;
+    if (j == 0) vmax = best;
+    const float p = expf(best - vmax);
+    den += p;
+    if (lane == j % 64) { myval = p; idx[(size_t)t * top + j] = bi; }
+    if (lane == 0) z[bi] = -INFINITY;
+    __syncthreads();
   }
+  if (lane < top) wt[(size_t)t * top + lane] = myval / den;
 }
 
 __global__ void __launch_bounds__(1024)
@@ -86,16 +75,10 @@ moe_combine_kernel(const float* __restrict__ y, const int32_t* __restrict__ inv,
 
 #define LAUNCH_OK() (hipGetLastError() == hipSuccess ? SSD_OK : SSD_ERR_LAUNCH)
 
-extern "C" int ssd_moe_route(const void* h_rows, const void* w_router, int32_t* idx, float* weights, int T, int W, int E, int top,
-                             int f32, void* stream) {
-  if (!h_rows || !w_router || !idx || !weights) return SSD_ERR_ARG;
-  if (T <= 0 || W <= 0 || E <= 0 || E > MOE_MAX_E || top <= 0 || top > E || top > MOE_MAX_TOP) return SSD_ERR_SHAPE;
-  if (f32)
-    hipLaunchKernelGGL(moe_route_kernel<float>, dim3(T), dim3(256), E * sizeof(float), (hipStream_t)stream, (const float*)h_rows,
-                       (const float*)w_router, idx, weights, W, E, top);
-  else
-    hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(T), dim3(256), E * sizeof(float), (hipStream_t)stream, (const bf16_t*)h_rows,
-                       (const bf16_t*)w_router, idx, weights, W, E, top);
+extern "C" int ssd_moe_route(const float* logits, int32_t* idx, float* weights, int T, int E, int top, void* stream) {
+  if (!logits || !idx || !weights) return SSD_ERR_ARG;
+  if (T <= 0 || E <= 0 || E > MOE_MAX_E || top <= 0 || top > E || top > MOE_MAX_TOP) return SSD_ERR_SHAPE;
+  hipLaunchKernelGGL(moe_route_kernel, dim3(T), dim3(64), E * sizeof(float), (hipStream_t)stream, logits, idx, weights, E, top);
   return LAUNCH_OK();
 }
 

@@ -3,7 +3,7 @@ a routed (mixture-of-experts) feed-forward with a shared expert, and a span of l
 
 Per layer run the launch list is
     rmsnorm_res32 (+ the embedding output before a repeated pass) -> fused [q | k | v | gate] GEMM -> diffattn_store (q / k norms,
-    KV store, gate sigmoid) -> diffattn_paged -> o GEMM -> rmsnorm_add_res32 -> rmsnorm_res32 -> moe_route -> moe_plan ->
+    KV store, gate sigmoid) -> diffattn_paged -> o GEMM -> rmsnorm_add_res32 -> rmsnorm_res32 -> router GEMM -> moe_route -> moe_plan ->
     grouped up GEMM (relu^2 epilogue) -> grouped down GEMM -> shared up / down GEMMs -> moe_combine -> rmsnorm_add_res32
 over pre-allocated buffers (nothing is allocated during a forward: it can be captured in a hipGraph like the other decoders).
 Same interface as ssd_amd.model.HipDecoder towards the ModelRunner: forward / compute_logits / argmax / full_logits / alloc_kv.
@@ -66,6 +66,7 @@ class HipFatulix:
             top = max(m.top for m in mlps)
             self.r_idx = z(T * top, dtype=torch.int32)
             self.r_wt = z(T * top)
+            self.r_z = z(T * max(m.experts for m in mlps))
             self.r_off = z(max(m.experts for m in mlps) + 1, dtype=torch.int32)
             self.r_perm = z(T * top, dtype=torch.int32)
             self.r_inv = z(T * top, dtype=torch.int32)
@@ -169,7 +170,8 @@ class HipFatulix:
         """hn (normalised rows) -> y (fp32 feed-forward output rows)."""
         w, f, W = self.w, self.f32, self.W
         ml, p = self.cfg.layers[li].mlp, f"l{li}.mlp."
-        H.moe_route(self.hn, w[p + "router"], self.r_idx, self.r_wt, T, W, ml.experts, ml.top, f)
+        H.gemm_rows(self.hn, w[p + "router"], self.r_z, T, ml.experts, W, f)
+        H.moe_route(self.r_z, self.r_idx, self.r_wt, T, ml.experts, ml.top)
         H.moe_plan(self.r_idx, T, ml.top, ml.experts, self.r_off, self.r_perm, self.r_inv)
         H.gemm_rows_grouped(self.hn, w[p + "up"], self.act, self.r_off, ml.experts, T * ml.top, ml.ff, W, f, H.GR_RELU2,
                             row_idx=self.r_perm, idx_div=ml.top)

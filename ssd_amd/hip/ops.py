@@ -426,8 +426,8 @@ def diffattn_paged(q, k_cache, v_cache, gate, block_tables, max_blocks, position
                                              out_scale, eps, _p(out_rows), int(f32), _stream()), "ssd_diffattn_paged")
 
 
-def moe_route(h, w_router, idx, weights, T: int, W: int, E: int, top: int, f32: bool):
-    _check(load_library().ssd_moe_route(_p(h), _p(w_router), _p(idx), _p(weights), T, W, E, top, int(f32), _stream()), "ssd_moe_route")
+def moe_route(logits, idx, weights, T: int, E: int, top: int):
+    _check(load_library().ssd_moe_route(_p(logits), _p(idx), _p(weights), T, E, top, _stream()), "ssd_moe_route")
 
 
 def moe_plan(idx, T: int, top: int, E: int, offsets, perm, inv):

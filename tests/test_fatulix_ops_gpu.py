@@ -109,7 +109,9 @@ def test_route_plan_combine(f32, E, top):
     h, wr = _rand((T, W), f32, g), _rand((E, W), f32, g, 1 / math.sqrt(W))
     idx = torch.zeros(T, top, dtype=torch.int32, device=DEV)
     wt = torch.zeros(T, top, device=DEV)
-    H.moe_route(h, wr, idx, wt, T, W, E, top, f32)
+    zl = torch.zeros(T, E, device=DEV)
+    H.gemm_rows(h, wr, zl, T, E, W, f32)
+    H.moe_route(zl, idx, wt, T, E, top)
     z = h.double() @ wr.double().T
     val, ref_idx = z.topk(top, dim=-1)
     assert torch.equal(idx.long(), ref_idx)                      # random logits: no close calls

@@ -383,6 +383,13 @@ int ssd_rmsnorm_res32(void* x, const void* add, const void* weight, float eps, v
                       int f32, void* stream);
 /* x += weight * y / sqrt(mean(y^2) + eps): the norm AFTER a sublayer and the residual sum; y fp32 [T][W]. */
 int ssd_rmsnorm_add_res32(const void* y, const void* weight, float eps, void* x, int T, int W, int f32, void* stream);
+/* The tail of a sandwich sublayer in one launch: y = y_rows (fp32 [T][W]) or, when y_rows is NULL, the routed mix
+ * sum_j weights[t][j] * ydn_rows[inv[t*top+j]] (+ shared_rows[t]) (written to y_scratch); x += post_weight * rms(y); then, with
+ * next_weight / next_out: x += next_add (optional), next_out = next_weight * rms(x).  Same arithmetic as ssd_moe_combine +
+ * ssd_rmsnorm_add_res32 + ssd_rmsnorm_res32. */
+int ssd_sandwich_tail(const void* y_rows, const void* ydn_rows, const int32_t* inv, const float* weights, const void* shared_rows,
+                      int top, void* y_scratch, const void* post_weight, float eps, void* x, const void* next_add,
+                      const void* next_weight, void* next_out, int T, int W, int f32, void* stream);
 /* fp32 rows [rows][ld_src] -> bf16 rows [rows][ld_dst]; columns cols .. ld_dst-1 of dst are set to -inf. */
 int ssd_rows_f32_to_bf16(const void* src, void* dst, int rows, int cols, long ld_src, long ld_dst, void* stream);
 
@@ -403,11 +410,13 @@ int ssd_diffattn_store(const void* qkvg_rows, const void* q_norm_w, const void* 
 /* out[t][h] = out_scale * gate[t][h] * rms_noweight(a_1 - lambda * a_2), a_m = softmax(scale * q_m . k_m) v over keys
  * 0 .. positions[t] of the token's sequence (cu_q int32 [B+1] row ranges, or q_per_seq rows per sequence when cu_q is NULL).
  * context_lens int32 [B] (keys each sequence holds) and max_q (most rows of one sequence) are optional (NULL / 0); with them, bf16,
- * D % 8 == 0, D <= 128, Dv % 16 == 0, Dv <= 128 and block_size % 32 == 0 the MFMA form runs, else the fp32 scalar form. */
+ * D % 8 == 0, D <= 128, Dv % 16 == 0, Dv <= 128 and block_size % 32 == 0 the MFMA form runs, else the fp32 scalar form.
+ * workspace (optional, fp32, workspace_bytes) + ctx_hint (host-side bound of the context lengths): decoding rows cut their keys
+ * over up to 16 workgroups per (sequence, kv head); 4160 floats per (sequence, kv head, slice). */
 int ssd_diffattn_paged(const void* q_rows, const void* k_cache, const void* v_cache, const void* gate, const int32_t* block_tables,
                        int max_blocks, const int64_t* positions, const int32_t* context_lens, const int32_t* cu_q, int q_per_seq,
                        int max_q, int B, int T, int H, int G, int D, int Dv, int block_size, float scale, float lambda, float out_scale,
-                       float eps, void* out_rows, int f32, void* stream);
+                       float eps, void* out_rows, int f32, void* workspace, long workspace_bytes, int ctx_hint, void* stream);
 
 /* Routed feed-forward (csrc/moe.hip): from the router's fp32 logits [T][E] (ssd_gemm_rows, fp32 rows out) the `top` largest per token,
  * softmax over the chosen ones;

@@ -195,7 +195,8 @@ diffattn_paged_kernel(const T* __restrict__ q, const T* __restrict__ kc, const T
 // The k slots of the second product are the keys in the order the first product's fragments hold them, so no data moves between lanes.
 // tile mode  (prompt portions): workgroup = 4 waves = 64 consecutive rows of one sequence, every wave scans keys 0 .. its last row's position.
 // split mode (<= 16 rows per sequence: decoding): the 4 waves share the rows and split the keys; partial (max, sum, O) merge in LDS
-//            in wave order.
+//            in wave order.  With a workspace the keys are first cut into slices over blockIdx.z; a one-wave merge kernel per
+//            (sequence, kv head) then sums the slices in order.
 // Keys past a row's position are masked by select (whatever the cache holds there); V of keys past the sequence's length is zeroed.
 // ---------------------------------------------------------------------------------------------------------------------
 constexpr int DM_KS = 4, DM_DVT = 8;
@@ -203,12 +204,38 @@ constexpr int DM_KS = 4, DM_DVT = 8;
 __device__ __forceinline__ float quad_max(float v) { v = fmaxf(v, __shfl_xor(v, 16, 64)); return fmaxf(v, __shfl_xor(v, 32, 64)); }
 __device__ __forceinline__ float quad_sum(float v) { v += __shfl_xor(v, 16, 64); return v + __shfl_xor(v, 32, 64); }
 
+constexpr int DM_WS_SLOT = 64 + 2 * DM_DVT * 64 * 4;      // floats per (sequence, kv head, key slice): max / sum rows, then the O fragments
+
+// Combine the maps, norm over the head's values, scale, gate; lane (row r, values i*16 + qd*4 ..+3) holds acc[m][i][0..3].
+__device__ __forceinline__ void diff_finalize(f32x4_t (&acc)[2][DM_DVT], const float (&ls)[2], int DVT, int Dv, float lambda,
+                                              float out_scale, float gate, float eps, bool valid, bf16_t* orow) {
+  const float i1 = 1.0f / ls[0], i2 = lambda / ls[1];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < DM_DVT; ++i)
+    if (i < DVT) {
+      acc[0][i] = acc[0][i] * i1 - acc[1][i] * i2;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += acc[0][i][e] * acc[0][i][e];
+    }
+  ss = quad_sum(ss);
+  const float rn = out_scale * gate / sqrtf(ss / (float)Dv + eps);
+  if (valid) {
+#pragma unroll
+    for (int i = 0; i < DM_DVT; ++i)
+      if (i < DVT) {
+        const u32x2_t o = {pack_bf2(acc[0][i][0] * rn, acc[0][i][1] * rn), pack_bf2(acc[0][i][2] * rn, acc[0][i][3] * rn)};
+        *reinterpret_cast<u32x2_t*>(orow + i * 16) = o;
+      }
+  }
+}
+
 __global__ void __launch_bounds__(256)
 diffattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vt,
                      const float* __restrict__ gate, const int32_t* __restrict__ bt, int max_blocks,
                      const int64_t* __restrict__ positions, const int32_t* __restrict__ ctx_lens, const int32_t* __restrict__ cu_q,
                      int q_per_seq, int B, int H, int G, int D, int Dv, int bs, float scale, float lambda, float out_scale, float eps,
-                     bf16_t* __restrict__ out, int split) {
+                     bf16_t* __restrict__ out, int split, int nsplit, float* __restrict__ ws) {
   extern __shared__ float smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, qd = lane >> 4;
   const int g = blockIdx.y, R = H / G;
@@ -264,7 +291,13 @@ diffattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc
 
   const int nsteps = (maxpos >> 5) + 1;
   int s_begin = 0, s_end = nsteps;
-  if (split) { const int per = (nsteps + 3) >> 2; s_begin = wave * per; s_end = min(nsteps, s_begin + per); }
+  if (split) {        // this workgroup's slice of the steps (all of them without a grid split), cut over the four waves
+    const int per_wg = (nsteps + nsplit - 1) / nsplit;
+    const int g_begin = min(nsteps, (int)blockIdx.z * per_wg), g_end = min(nsteps, g_begin + per_wg);
+    const int per = (g_end - g_begin + 3) >> 2;
+    s_begin = min(g_end, g_begin + wave * per);
+    s_end = min(g_end, s_begin + per);
+  }
 
   for (int st = s_begin; st < s_end; ++st) {
     const int k0 = st << 5;
@@ -361,6 +394,7 @@ diffattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc
 #pragma unroll
       for (int i = 0; i < DM_DVT; ++i) acc[m][i] *= f;
       ls[m] = L;
+      mx[m] = M;
     }
     for (int w = 1; w < 4; ++w) {
       if (wave == w) {
@@ -383,27 +417,62 @@ diffattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc
     if (wave != 0) return;
   }
 
-  // ---- combine the maps, norm over the head's values, scale, gate; lane (row r, values i*16 + qd*4 ..+3) ----
-  const float i1 = 1.0f / ls[0], i2 = lambda / ls[1];
-  float ss = 0.f;
+  if (nsplit > 1) {
+    // ---- this workgroup scanned one slice of the keys: leave (max, sum, O) for the merge kernel, in register layout ----
+    const size_t slot = ((size_t)b * G + g) * nsplit + blockIdx.z;
+    float* wml = ws + slot * DM_WS_SLOT;
+    if (qd == 0) {
 #pragma unroll
-  for (int i = 0; i < DM_DVT; ++i)
-    if (i < DVT) {
-      acc[0][i] = acc[0][i] * i1 - acc[1][i] * i2;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) ss += acc[0][i][e] * acc[0][i][e];
+      for (int m = 0; m < 2; ++m) { wml[(m * 2 + 0) * 16 + r] = mx[m]; wml[(m * 2 + 1) * 16 + r] = ls[m]; }
     }
-  ss = quad_sum(ss);
-  const float rn = out_scale * gate[(size_t)token * H + head] / sqrtf(ss / (float)Dv + eps);
-  if (valid) {
-    bf16_t* orow = out + ((size_t)token * H + head) * Dv + qd * 4;
+    f32x4_t* wacc = reinterpret_cast<f32x4_t*>(wml + 64);
 #pragma unroll
-    for (int i = 0; i < DM_DVT; ++i)
-      if (i < DVT) {
-        const u32x2_t o = {pack_bf2(acc[0][i][0] * rn, acc[0][i][1] * rn), pack_bf2(acc[0][i][2] * rn, acc[0][i][3] * rn)};
-        *reinterpret_cast<u32x2_t*>(orow + i * 16) = o;
-      }
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+      for (int i = 0; i < DM_DVT; ++i)
+        if (i < DVT) wacc[(m * DM_DVT + i) * 64 + lane] = acc[m][i];
+    return;
   }
+  diff_finalize(acc, ls, DVT, Dv, lambda, out_scale, gate[(size_t)token * H + head], eps, valid,
+                out + ((size_t)token * H + head) * Dv + qd * 4);
+}
+
+// The second pass of a key-split decode: one wave per (sequence, kv head) sums the slices' partials in slice order and finishes the rows.
+__global__ void __launch_bounds__(64)
+diffattn_merge_kernel(const float* __restrict__ ws, int nsplit, const float* __restrict__ gate, const int32_t* __restrict__ cu_q,
+                      int q_per_seq, int H, int G, int Dv, float lambda, float out_scale, float eps, bf16_t* __restrict__ out) {
+  const int lane = threadIdx.x, r = lane & 15, qd = lane >> 4;
+  const int b = blockIdx.x, g = blockIdx.y, R = H / G, DVT = Dv >> 4;
+  const int tok0 = cu_q ? cu_q[b] : b * q_per_seq;
+  const int qb = cu_q ? cu_q[b + 1] - cu_q[b] : q_per_seq;
+  const bool valid = r < qb * R;
+  const int rr = valid ? r : 0;
+  const int token = tok0 + rr / R, head = g * R + rr % R;
+  const float* base = ws + ((size_t)b * G + g) * nsplit * DM_WS_SLOT;
+  float M[2] = {-INFINITY, -INFINITY}, ls[2] = {0.f, 0.f};
+  for (int sidx = 0; sidx < nsplit; ++sidx)
+#pragma unroll
+    for (int m = 0; m < 2; ++m) M[m] = fmaxf(M[m], base[(size_t)sidx * DM_WS_SLOT + (m * 2 + 0) * 16 + r]);
+  f32x4_t acc[2][DM_DVT];
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int i = 0; i < DM_DVT; ++i) acc[m][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int sidx = 0; sidx < nsplit; ++sidx) {
+    const float* wml = base + (size_t)sidx * DM_WS_SLOT;
+    const f32x4_t* wacc = reinterpret_cast<const f32x4_t*>(wml + 64);
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      const float ms = wml[(m * 2 + 0) * 16 + r];
+      const float f = ms == -INFINITY ? 0.f : __expf(ms - M[m]);
+      ls[m] += wml[(m * 2 + 1) * 16 + r] * f;
+#pragma unroll
+      for (int i = 0; i < DM_DVT; ++i)
+        if (i < DVT) acc[m][i] += wacc[(m * DM_DVT + i) * 64 + lane] * f;
+    }
+  }
+  diff_finalize(acc, ls, DVT, Dv, lambda, out_scale, gate[(size_t)token * H + head], eps, valid,
+                out + ((size_t)token * H + head) * Dv + qd * 4);
 }
 
 }  // namespace
@@ -430,7 +499,7 @@ extern "C" int ssd_diffattn_paged(const void* q_rows, const void* k_cache, const
                                   const int32_t* block_tables, int max_blocks, const int64_t* positions, const int32_t* context_lens,
                                   const int32_t* cu_q, int q_per_seq, int max_q, int B, int T, int H, int G, int D, int Dv,
                                   int block_size, float scale, float lambda, float out_scale, float eps, void* out_rows, int f32,
-                                  void* stream) {
+                                  void* workspace, long workspace_bytes, int ctx_hint, void* stream) {
   if (!q_rows || !k_cache || !v_cache || !gate || !block_tables || !positions || !out_rows) return SSD_ERR_ARG;
   if (T <= 0 || B <= 0 || H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || Dv > 64 * DA_MAXV || block_size <= 0 || max_blocks <= 0)
     return SSD_ERR_SHAPE;
@@ -441,9 +510,24 @@ extern "C" int ssd_diffattn_paged(const void* q_rows, const void* k_cache, const
     const int split = max_q * R <= 16 ? 1 : 0;
     const int gx = split ? B : ((long)T * R + 63) / 64 + B;
     const size_t lds_m = split ? (size_t)(4 * 2 * 2 * 16 + 2 * (Dv / 16) * 64 * 4) * 4 : 0;
-    hipLaunchKernelGGL(diffattn_mfma_kernel, dim3(gx, G), dim3(256), lds_m, (hipStream_t)stream, (const bf16_t*)q_rows,
+    // decoding rows of few sequences: cut the keys over more workgroups (a launch of B * G workgroups leaves most of the chip idle)
+    // when the caller gave a workspace and says the contexts are long; every wave keeps at least 4 steps of 32 keys
+    int nsplit = 1;
+    if (split && workspace && ctx_hint > 0) {
+      nsplit = 256 / (B * G);
+      const int by_len = ctx_hint / (32 * 4 * 4);
+      if (nsplit > by_len) nsplit = by_len;
+      if (nsplit > 16) nsplit = 16;
+      while (nsplit > 1 && (long)B * G * nsplit * DM_WS_SLOT * 4 > workspace_bytes) --nsplit;
+      if (nsplit < 1) nsplit = 1;
+    }
+    hipLaunchKernelGGL(diffattn_mfma_kernel, dim3(gx, G, nsplit), dim3(256), lds_m, (hipStream_t)stream, (const bf16_t*)q_rows,
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, (const float*)gate, block_tables, max_blocks, positions,
-                       context_lens, cu_q, q_per_seq, B, H, G, D, Dv, block_size, scale, lambda, out_scale, eps, (bf16_t*)out_rows, split);
+                       context_lens, cu_q, q_per_seq, B, H, G, D, Dv, block_size, scale, lambda, out_scale, eps, (bf16_t*)out_rows, split,
+                       nsplit, (float*)workspace);
+    if (nsplit > 1)
+      hipLaunchKernelGGL(diffattn_merge_kernel, dim3(B, G), dim3(64), 0, (hipStream_t)stream, (const float*)workspace, nsplit,
+                         (const float*)gate, cu_q, q_per_seq, H, G, Dv, lambda, out_scale, eps, (bf16_t*)out_rows);
     return LAUNCH_OK();
   }
   const size_t lds = (size_t)(2 * D + 4 * 2 * 64) * 4 + 4 * 64 * 8 + (size_t)(4 * 2 * Dv + 16 + 4) * 4 + 8;

@@ -4,6 +4,7 @@
 //  * ssd_rmsnorm_res32      y = w * x / sqrt(mean(x^2) + eps) from the fp32 residual to GEMM-input rows; optionally x += add first
 //                           (the re-injected embedding before a repeated pass) and a row gather (logit rows)
 //  * ssd_rmsnorm_add_res32  x += w * rms(y) for the fp32 sublayer output y
+//  * ssd_sandwich_tail      (routed mix ->) post-norm + residual sum -> (re-injection ->) the next sublayer's pre-norm, one launch
 //  * ssd_rows_f32_to_bf16   fp32 rows -> bf16 rows with their own row stride, padding columns = -inf (fp32 logits for the bf16 sampling kernels)
 // All reductions are fp32, one workgroup of 256 threads per row, a fixed summation order per row (independent of the batch).
 // `f32` selects the element type of weights and of GEMM-input rows: 0 = bf16, 1 = fp32.
@@ -74,9 +75,52 @@ rmsnorm_add_res32_kernel(const float* __restrict__ y, const T* __restrict__ w, f
   for (int c = threadIdx.x; c < W; c += 256) xr[c] += yr[c] * r * ldf<T>(w + c);
 }
 
+// The whole tail of a sandwich sublayer for one token row per workgroup:
+//   y = the sublayer's fp32 output row, or the routed feed-forward's mix  sum_j weights[j] * ydn[inv[t * top + j]] (+ shared[t])
+//   x += w_post * rms(y);   then, if a next sublayer follows:  x += next_add (the re-injected embedding before a repeated pass),
+//   next_out = w_next * rms(x)  -- the input rows of the next sublayer's first GEMM.
+// Three launches (mix, post-norm + residual sum, next pre-norm) in one; the same arithmetic in the same order as the separate kernels.
+template <typename T>
+__global__ void __launch_bounds__(256)
+sandwich_tail_kernel(const float* __restrict__ y, const float* __restrict__ ydn, const int32_t* __restrict__ inv,
+                     const float* __restrict__ wt, const float* __restrict__ shared, int top, float* __restrict__ ytmp,
+                     const T* __restrict__ w_post, float eps, float* __restrict__ x, const float* __restrict__ next_add,
+                     const T* __restrict__ w_next, T* __restrict__ next_out, int W) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  float* xr = x + (size_t)t * W;
+  const float* yr = y ? y + (size_t)t * W : ytmp + (size_t)t * W;
+  float ss = 0.f;
+  if (y) {
+    for (int c = threadIdx.x; c < W; c += 256) { const float v = yr[c]; ss += v * v; }
+  } else {
+    float* yw = ytmp + (size_t)t * W;
+    for (int c = threadIdx.x; c < W; c += 256) {
+      float v = 0.f;
+      for (int j = 0; j < top; ++j) v = fmaf(wt[(size_t)t * top + j], ydn[(size_t)inv[(size_t)t * top + j] * W + c], v);
+      if (shared) v += shared[(size_t)t * W + c];
+      yw[c] = v;                    // read back below by the thread that wrote it
+      ss += v * v;
+    }
+  }
+  ss = block_sum_256(ss, red);
+  const float r = 1.0f / sqrtf(ss / (float)W + eps);
+  float s2 = 0.f;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    float v = xr[c] + yr[c] * r * ldf<T>(w_post + c);
+    if (next_add) v += next_add[(size_t)t * W + c];
+    xr[c] = v;
+    s2 += v * v;
+  }
+  if (!w_next) return;
+  s2 = block_sum_256(s2, red);
+  const float r2 = 1.0f / sqrtf(s2 / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += 256) stf<T>(next_out + (size_t)t * W + c, xr[c] * r2 * ldf<T>(w_next + c));
+}
+
 __global__ void rows_f32_to_bf16_kernel(const float* __restrict__ src, bf16_t* __restrict__ dst, int cols, long ld_src, long ld_dst) {
   const long r = blockIdx.x;
-  for (int c = threadIdx.x; c < ld_dst; c += blockDim.x) dst[r * ld_dst + c] = c < cols ? (bf16_t)f2bf(src[r * ld_src + c]) : (bf16_t)0xff80u;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < ld_dst; c += gridDim.y * blockDim.x) dst[r * ld_dst + c] = c < cols ? (bf16_t)f2bf(src[r * ld_src + c]) : (bf16_t)0xff80u;
 }
 
 }  // namespace
@@ -125,7 +169,27 @@ extern "C" int ssd_rmsnorm_add_res32(const void* y, const void* weight, float ep
 extern "C" int ssd_rows_f32_to_bf16(const void* src, void* dst, int rows, int cols, long ld_src, long ld_dst, void* stream) {
   if (!src || !dst) return SSD_ERR_ARG;
   if (rows <= 0 || cols <= 0 || ld_src < cols || ld_dst < cols) return SSD_ERR_SHAPE;
-  hipLaunchKernelGGL(rows_f32_to_bf16_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, (const float*)src, (bf16_t*)dst, cols,
+  const int chunks = (int)((ld_dst + 2047) / 2048);
+  hipLaunchKernelGGL(rows_f32_to_bf16_kernel, dim3(rows, chunks), dim3(256), 0, (hipStream_t)stream, (const float*)src, (bf16_t*)dst, cols,
                      ld_src, ld_dst);
+  return LAUNCH_OK();
+}
+
+extern "C" int ssd_sandwich_tail(const void* y_rows, const void* ydn_rows, const int32_t* inv, const float* weights,
+                                 const void* shared_rows, int top, void* y_scratch, const void* post_weight, float eps, void* x,
+                                 const void* next_add, const void* next_weight, void* next_out, int T, int W, int f32, void* stream) {
+  if (!post_weight || !x) return SSD_ERR_ARG;
+  if (!y_rows && (!ydn_rows || !inv || !weights || !y_scratch || top <= 0)) return SSD_ERR_ARG;
+  if ((next_weight == nullptr) != (next_out == nullptr) || (next_add && !next_weight)) return SSD_ERR_ARG;
+  if (T <= 0 || W <= 0) return SSD_ERR_SHAPE;
+  if (f32)
+    hipLaunchKernelGGL(sandwich_tail_kernel<float>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)y_rows,
+                       (const float*)ydn_rows, inv, weights, (const float*)shared_rows, top, (float*)y_scratch,
+                       (const float*)post_weight, eps, (float*)x, (const float*)next_add, (const float*)next_weight, (float*)next_out, W);
+  else
+    hipLaunchKernelGGL(sandwich_tail_kernel<bf16_t>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)y_rows,
+                       (const float*)ydn_rows, inv, weights, (const float*)shared_rows, top, (float*)y_scratch,
+                       (const bf16_t*)post_weight, eps, (float*)x, (const float*)next_add, (const bf16_t*)next_weight,
+                       (bf16_t*)next_out, W);
   return LAUNCH_OK();
 }

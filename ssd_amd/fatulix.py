@@ -2,9 +2,10 @@
 a routed (mixture-of-experts) feed-forward with a shared expert, and a span of layers that runs several passes with the same weights.
 
 Per layer run the launch list is
-    rmsnorm_res32 (+ the embedding output before a repeated pass) -> fused [q | k | v | gate] GEMM -> diffattn_store (q / k norms,
-    KV store, gate sigmoid) -> diffattn_paged -> o GEMM -> rmsnorm_add_res32 -> rmsnorm_res32 -> router GEMM -> moe_route -> moe_plan ->
-    grouped up GEMM (relu^2 epilogue) -> grouped down GEMM -> shared up / down GEMMs -> moe_combine -> rmsnorm_add_res32
+    fused [q | k | v | gate] GEMM -> diffattn_store (q / k norms, KV store, gate sigmoid) -> diffattn_paged -> o GEMM ->
+    sandwich_tail (post-norm + residual sum + the feed-forward's pre-norm) -> router GEMM -> moe_route -> moe_plan -> grouped up
+    GEMM (relu^2 epilogue) -> grouped down GEMM -> shared up / down GEMMs -> sandwich_tail (routed mix + post-norm + residual sum +
+    the embedding output before a repeated pass + the next run's pre-norm)
 over pre-allocated buffers (nothing is allocated during a forward: it can be captured in a hipGraph like the other decoders).
 Same interface as ssd_amd.model.HipDecoder towards the ModelRunner: forward / compute_logits / argmax / full_logits / alloc_kv.
 
@@ -62,6 +63,7 @@ class HipFatulix:
         self.q = z(T * max(m.heads * 2 * m.dim for m in mix), dtype=el)
         self.gate = z(T * max(m.heads for m in mix))
         self.att = z(T * max(m.heads * m.vdim for m in mix), dtype=el)
+        self.att_ws = z(256 * 4160)           # key-slice partials of the decode attention (csrc/attention_diff.hip): <= 256 slices in flight
         if mlps:
             top = max(m.top for m in mlps)
             self.r_idx = z(T * top, dtype=torch.int32)
@@ -163,11 +165,13 @@ class HipFatulix:
                          T, m.heads, m.kv_heads, m.dim, m.vdim, self.block_size, f)
         H.diffattn_paged(self.q, kc, vc, self.gate, meta.block_tables, self.max_blocks, positions, meta.B, T, m.heads, m.kv_heads,
                          m.dim, m.vdim, self.block_size, m.scale, self.lam[li], 1.0 - m.diff, cfg.rms_norm_eps, self.att, f,
-                         cu_q=meta.cu_q, q_per_seq=meta.q_per_seq, context_lens=meta.context_lens, max_q=meta.max_q)
+                         cu_q=meta.cu_q, q_per_seq=meta.q_per_seq, context_lens=meta.context_lens, max_q=meta.max_q,
+                         workspace=self.att_ws, ctx_hint=meta.ctx_hint)
         H.gemm_rows(self.att, w[p + "o"], self.y, T, self.W, m.heads * m.vdim, f)
 
-    def launch_mlp(self, li: int, T: int) -> None:
-        """hn (normalised rows) -> y (fp32 feed-forward output rows)."""
+    def launch_mlp(self, li: int, T: int, combine: bool = True) -> None:
+        """hn (normalised rows) -> y (fp32 feed-forward output rows); combine=False leaves the experts' rows in ydn / ysh for the
+        fused tail (ssd_sandwich_tail)."""
         w, f, W = self.w, self.f32, self.W
         ml, p = self.cfg.layers[li].mlp, f"l{li}.mlp."
         H.gemm_rows(self.hn, w[p + "router"], self.r_z, T, ml.experts, W, f)
@@ -179,7 +183,8 @@ class HipFatulix:
         if ml.shared_ff:
             H.gemm_rows(self.hn, w[p + "shared.up"], self.sact, T, ml.shared_ff, W, f, H.GR_RELU2)
             H.gemm_rows(self.sact, w[p + "shared.down"], self.ysh, T, W, ml.shared_ff, f)
-        H.moe_combine(self.ydn, self.r_inv, self.r_wt, self.ysh if ml.shared_ff else None, self.y, T, ml.top, W)
+        if combine:
+            H.moe_combine(self.ydn, self.r_inv, self.r_wt, self.ysh if ml.shared_ff else None, self.y, T, ml.top, W)
 
     def forward(self, input_ids: torch.Tensor, positions: torch.Tensor, T: int, meta: AttnMeta) -> None:
         """Runs every layer run over the T token rows; leaves the fp32 residual rows in self.x."""
@@ -187,9 +192,35 @@ class HipFatulix:
         assert T <= self.max_tokens and meta.mode == H.MODE_CAUSAL and (meta.cu_q is not None or meta.q_per_seq > 0)
         eps = cfg.rms_norm_eps
         H.embed_res32(input_ids, w["embed"], self.x, self.x0, T, W, f)
+        if self.tap_residuals is not None:
+            return self._forward_unfused(positions, T, meta)
+        # fused tails: every sublayer's post-norm + residual sum also writes the NEXT sublayer's normalised input (one launch; the
+        # routed mix rides along), so only the first layer run has a norm launch of its own
+        H.rmsnorm_res32(self.x, w[f"l{self.runs[0][0]}.norm1"], eps, self.hn, T, W, f)
+        for run, (li, ps) in enumerate(self.runs):
+            p, ml = f"l{li}.", cfg.layers[li].mlp
+            nxt = {}
+            if run + 1 < len(self.runs):
+                nli, nps = self.runs[run + 1]
+                nxt = dict(next_weight=w[f"l{nli}.norm1"], next_out=self.hn,
+                           next_add=self.x0 if (nps > 0 and nli == cfg.loop_start) else None)     # the embedding output re-enters
+            self.launch_mixer(run, li, T, positions, meta)
+            if ml is None:
+                H.sandwich_tail(w[p + "norm1b"], eps, self.x, T, W, f, y=self.y, **nxt)
+                continue
+            H.sandwich_tail(w[p + "norm1b"], eps, self.x, T, W, f, y=self.y, next_weight=w[p + "norm2"], next_out=self.hn)
+            self.launch_mlp(li, T, combine=False)
+            H.sandwich_tail(w[p + "norm2b"], eps, self.x, T, W, f, ydn=self.ydn, inv=self.r_inv, weights=self.r_wt,
+                            shared=self.ysh if ml.shared_ff else None, top=ml.top, y_scratch=self.y, **nxt)
+
+    def _forward_unfused(self, positions, T: int, meta: AttnMeta) -> None:
+        """The same forward with one launch per step (norm, mix, post-norm + sum) and a copy of the residual rows after every layer
+        run, before whatever precedes the next run (tests)."""
+        cfg, w, f, W = self.cfg, self.w, self.f32, self.W
+        eps = cfg.rms_norm_eps
         for run, (li, ps) in enumerate(self.runs):
             p = f"l{li}."
-            again = self.x0 if (ps > 0 and li == cfg.loop_start) else None      # the embedding output re-enters before a repeated pass
+            again = self.x0 if (ps > 0 and li == cfg.loop_start) else None
             H.rmsnorm_res32(self.x, w[p + "norm1"], eps, self.hn, T, W, f, add=again)
             self.launch_mixer(run, li, T, positions, meta)
             H.rmsnorm_add_res32(self.y, w[p + "norm1b"], eps, self.x, T, W, f)
@@ -197,8 +228,7 @@ class HipFatulix:
                 H.rmsnorm_res32(self.x, w[p + "norm2"], eps, self.hn, T, W, f)
                 self.launch_mlp(li, T)
                 H.rmsnorm_add_res32(self.y, w[p + "norm2b"], eps, self.x, T, W, f)
-            if self.tap_residuals is not None:
-                self.tap_residuals.append(self.x[:T].clone())
+            self.tap_residuals.append(self.x[:T].clone())
 
     def compute_logits(self, T: int, gather: torch.Tensor | None = None, rows: int | None = None) -> int:
         """Final norm (optionally of the `gather` rows only) and the LM head: fp32 logits in logits32[:n], their bf16 rounding (row

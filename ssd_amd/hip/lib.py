@@ -113,13 +113,16 @@ SIGNATURES = {
     "ssd_embed_res32": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_void_p],
     "ssd_rmsnorm_res32": [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ssd_rmsnorm_add_res32": [c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ssd_sandwich_tail": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
+                          c_void_p, c_int, c_int, c_int, c_void_p],
     "ssd_rows_f32_to_bf16": [c_void_p, c_void_p, c_int, c_int, c_long, c_long, c_void_p],
     "ssd_gemm_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ssd_gemm_rows_grouped": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ssd_diffattn_store": [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                            c_int, c_int, c_int, c_int, c_void_p],
     "ssd_diffattn_paged": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                           c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_void_p, c_int, c_void_p],
+                           c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_void_p, c_int, c_void_p, c_long, c_int,
+                           c_void_p],
     "ssd_moe_route": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ssd_moe_plan": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
     "ssd_moe_combine": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],

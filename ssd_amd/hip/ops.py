@@ -394,6 +394,14 @@ def rmsnorm_add_res32(y, weight, eps: float, x, T: int, W: int, f32: bool):
     _check(load_library().ssd_rmsnorm_add_res32(_p(y), _p(weight), eps, _p(x), T, W, int(f32), _stream()), "ssd_rmsnorm_add_res32")
 
 
+def sandwich_tail(post_weight, eps: float, x, T: int, W: int, f32: bool, *, y=None, ydn=None, inv=None, weights=None, shared=None,
+                  top: int = 0, y_scratch=None, next_add=None, next_weight=None, next_out=None):
+    """x += post_weight * rms(y) [+ next_add]; next_out = next_weight * rms(x).  y: fp32 rows, or the routed mix of ydn (into y_scratch)."""
+    _check(load_library().ssd_sandwich_tail(_p(y), _p(ydn), _p(inv), _p(weights), _p(shared), top, _p(y_scratch), _p(post_weight), eps,
+                                            _p(x), _p(next_add), _p(next_weight), _p(next_out), T, W, int(f32), _stream()),
+           "ssd_sandwich_tail")
+
+
 def rows_f32_to_bf16(src, dst, rows: int, cols: int, ld_src: int, ld_dst: int):
     _check(load_library().ssd_rows_f32_to_bf16(_p(src), _p(dst), rows, cols, ld_src, ld_dst, _stream()), "ssd_rows_f32_to_bf16")
 
@@ -419,11 +427,14 @@ def diffattn_store(qkvg, q_norm_w, k_norm_w, eps: float, slots, q_out, gate_out,
 
 
 def diffattn_paged(q, k_cache, v_cache, gate, block_tables, max_blocks, positions, B, T, H, G, D, Dv, block_size, scale, lam,
-                   out_scale, eps, out_rows, f32: bool, cu_q=None, q_per_seq: int = 0, context_lens=None, max_q: int = 0):
+                   out_scale, eps, out_rows, f32: bool, cu_q=None, q_per_seq: int = 0, context_lens=None, max_q: int = 0, workspace=None,
+                   ctx_hint: int = 0):
     """context_lens + max_q given (and bf16, aligned head sizes, block_size % 32 == 0): the MFMA form; else the scalar fp32 form."""
     _check(load_library().ssd_diffattn_paged(_p(q), _p(k_cache), _p(v_cache), _p(gate), _p(block_tables), max_blocks, _p(positions),
                                              _p(context_lens), _p(cu_q), q_per_seq, max_q, B, T, H, G, D, Dv, block_size, scale, lam,
-                                             out_scale, eps, _p(out_rows), int(f32), _stream()), "ssd_diffattn_paged")
+                                             out_scale, eps, _p(out_rows), int(f32), _p(workspace),
+                                             workspace.numel() * workspace.element_size() if workspace is not None else 0, ctx_hint,
+                                             _stream()), "ssd_diffattn_paged")
 
 
 def moe_route(logits, idx, weights, T: int, E: int, top: int):

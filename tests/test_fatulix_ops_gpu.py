@@ -248,8 +248,46 @@ def test_diffattn_decode_rows_of_several_sequences(f32, Hh, G, D, Dv, bs):
     ctx = torch.tensor(lens, dtype=torch.int32, device=DEV)
     ref = _paged_ref(q, kc, vc, gate, bt, posd, torch.tensor(seq), Hh, G, D, Dv, bs, scale, lam, osc, eps)
     tol = dict(rtol=1e-4, atol=1e-4) if f32 else dict(rtol=2e-2, atol=2e-2)
-    for fast in (False, True):
+    ws = torch.zeros(256 * 4160, device=DEV)
+    for kw in ({}, dict(context_lens=ctx, max_q=2), dict(context_lens=ctx, max_q=2, workspace=ws, ctx_hint=4096)):
+        # the scalar form; the MFMA form (where the shape allows it in bf16); the same with the keys cut into slices over the grid
+        # (more slices than some sequences have steps: empty slices must merge as nothing)
         out = torch.zeros(T, Hh * Dv, dtype=el, device=DEV)
-        H.diffattn_paged(q, kc, vc, gate, bt, nblk, posd, B, T, Hh, G, D, Dv, bs, scale, lam, osc, eps, out, f32, cu_q=cu,
-                         **(dict(context_lens=ctx, max_q=2) if fast else {}))
+        H.diffattn_paged(q, kc, vc, gate, bt, nblk, posd, B, T, Hh, G, D, Dv, bs, scale, lam, osc, eps, out, f32, cu_q=cu, **kw)
         torch.testing.assert_close(out.double(), ref, **tol)
+
+
+@pytest.mark.parametrize("f32", MODES)
+@pytest.mark.parametrize("routed", [False, True])
+def test_sandwich_tail_equals_its_separate_launches(f32, routed):
+    from ssd_amd.hip import ops as H
+    g = torch.Generator().manual_seed(11)
+    T, W, top, eps = 7, 200, 3, 1e-5
+    el = _elem(f32)
+    wp, wn = _rand((W,), f32, g) + 1, _rand((W,), f32, g) + 1
+    x0 = torch.randn(T, W, generator=g).to(DEV)
+    add = torch.randn(T, W, generator=g).to(DEV)
+    ydn = torch.randn(T * top, W, generator=g).to(DEV)
+    sh = torch.randn(T, W, generator=g).to(DEV)
+    inv = torch.randperm(T * top, generator=g).to(torch.int32).to(DEV)
+    wt = torch.rand(T, top, generator=g).to(DEV)
+    y = torch.randn(T, W, generator=g).to(DEV)
+    # separate launches
+    xa = x0.clone()
+    if routed:
+        y = torch.zeros(T, W, device=DEV)
+        H.moe_combine(ydn, inv, wt, sh, y, T, top, W)
+    H.rmsnorm_add_res32(y, wp, eps, xa, T, W, f32)
+    na = torch.zeros(T, W, dtype=el, device=DEV)
+    H.rmsnorm_res32(xa, wn, eps, na, T, W, f32, add=add)
+    # one launch
+    xb, nb, scratch = x0.clone(), torch.zeros(T, W, dtype=el, device=DEV), torch.zeros(T, W, device=DEV)
+    src = dict(ydn=ydn, inv=inv, weights=wt, shared=sh, top=top, y_scratch=scratch) if routed else dict(y=y)
+    H.sandwich_tail(wp, eps, xb, T, W, f32, next_add=add, next_weight=wn, next_out=nb, **src)
+    torch.testing.assert_close(xb, xa, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(nb.float(), na.float(), **(dict(rtol=1e-6, atol=1e-6) if f32 else dict(rtol=1e-2, atol=1e-2)))
+    xc = x0.clone()                     # the last sublayer of a model: no next norm
+    H.sandwich_tail(wp, eps, xc, T, W, f32, **src)
+    xd = x0.clone()
+    H.rmsnorm_add_res32(y, wp, eps, xd, T, W, f32)
+    torch.testing.assert_close(xc, xd, rtol=1e-6, atol=1e-6)

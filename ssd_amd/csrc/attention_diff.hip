@@ -38,8 +38,9 @@ diffattn_store_kernel(const float* __restrict__ qkvg, const T* __restrict__ qw, 
   const int slot = slots[t];
   const long blk = slot >= 0 ? slot / bs : 0;
   const int off = slot >= 0 ? slot % bs : 0;
-  // q units 0 .. 2H-1, then k units 0 .. 2G-1: one wave per (head, map) vector of D values
-  for (int u = wave; u < 2 * H + 2 * G; u += 4) {
+  // q units 0 .. 2H-1, then k units 0 .. 2G-1: one wave per (head, map) vector of D values; the grid's y cuts the units (and the value /
+  // gate columns below) so that a single decoding token still spreads over many workgroups
+  for (int u = blockIdx.y * 4 + wave; u < 2 * H + 2 * G; u += 4 * gridDim.y) {
     const bool isq = u < 2 * H;
     const float* src = isq ? row + (size_t)u * D : row + Nq + (size_t)(u - 2 * H) * D;
     float ss = 0.f;
@@ -56,12 +57,13 @@ diffattn_store_kernel(const float* __restrict__ qkvg, const T* __restrict__ qw, 
     }
   }
   if (slot >= 0) {
-    for (int c = threadIdx.x; c < Nv; c += 256) {
+    for (int c = blockIdx.y * 256 + threadIdx.x; c < Nv; c += 256 * gridDim.y) {
       const int g = c / Dv, d = c % Dv;
       stf<T>(vc + (((size_t)blk * G + g) * Dv + d) * bs + off, row[Nq + Nk + c]);
     }
   }
-  for (int h = threadIdx.x; h < H; h += 256) gate_out[(size_t)t * H + h] = 1.0f / (1.0f + expf(-row[Nq + Nk + Nv + h]));
+  if (blockIdx.y == 0)
+    for (int h = threadIdx.x; h < H; h += 256) gate_out[(size_t)t * H + h] = 1.0f / (1.0f + expf(-row[Nq + Nk + Nv + h]));
 }
 
 template <typename T>
@@ -437,11 +439,13 @@ diffattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc
                 out + ((size_t)token * H + head) * Dv + qd * 4);
 }
 
-// The second pass of a key-split decode: one wave per (sequence, kv head) sums the slices' partials in slice order and finishes the rows.
-__global__ void __launch_bounds__(64)
+// The second pass of a key-split decode: one workgroup per (sequence, kv head); its 4 waves share the value tiles (wave w sums tiles
+// w, w + 4 of both maps over the slices, in slice order), the rows' mean squares meet in LDS, then every wave finishes its tiles.
+__global__ void __launch_bounds__(256)
 diffattn_merge_kernel(const float* __restrict__ ws, int nsplit, const float* __restrict__ gate, const int32_t* __restrict__ cu_q,
                       int q_per_seq, int H, int G, int Dv, float lambda, float out_scale, float eps, bf16_t* __restrict__ out) {
-  const int lane = threadIdx.x, r = lane & 15, qd = lane >> 4;
+  __shared__ float sss[4][16];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, qd = lane >> 4;
   const int b = blockIdx.x, g = blockIdx.y, R = H / G, DVT = Dv >> 4;
   const int tok0 = cu_q ? cu_q[b] : b * q_per_seq;
   const int qb = cu_q ? cu_q[b + 1] - cu_q[b] : q_per_seq;
@@ -453,11 +457,12 @@ diffattn_merge_kernel(const float* __restrict__ ws, int nsplit, const float* __r
   for (int sidx = 0; sidx < nsplit; ++sidx)
 #pragma unroll
     for (int m = 0; m < 2; ++m) M[m] = fmaxf(M[m], base[(size_t)sidx * DM_WS_SLOT + (m * 2 + 0) * 16 + r]);
-  f32x4_t acc[2][DM_DVT];
+  constexpr int PER = DM_DVT / 4;
+  f32x4_t acc[2][PER];
 #pragma unroll
   for (int m = 0; m < 2; ++m)
 #pragma unroll
-    for (int i = 0; i < DM_DVT; ++i) acc[m][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < PER; ++k) acc[m][k] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   for (int sidx = 0; sidx < nsplit; ++sidx) {
     const float* wml = base + (size_t)sidx * DM_WS_SLOT;
     const f32x4_t* wacc = reinterpret_cast<const f32x4_t*>(wml + 64);
@@ -467,12 +472,37 @@ diffattn_merge_kernel(const float* __restrict__ ws, int nsplit, const float* __r
       const float f = ms == -INFINITY ? 0.f : __expf(ms - M[m]);
       ls[m] += wml[(m * 2 + 1) * 16 + r] * f;
 #pragma unroll
-      for (int i = 0; i < DM_DVT; ++i)
-        if (i < DVT) acc[m][i] += wacc[(m * DM_DVT + i) * 64 + lane] * f;
+      for (int k = 0; k < PER; ++k) {
+        const int i = wave + 4 * k;
+        if (i < DVT) acc[m][k] += wacc[(m * DM_DVT + i) * 64 + lane] * f;
+      }
     }
   }
-  diff_finalize(acc, ls, DVT, Dv, lambda, out_scale, gate[(size_t)token * H + head], eps, valid,
-                out + ((size_t)token * H + head) * Dv + qd * 4);
+  const float i1 = 1.0f / ls[0], i2 = lambda / ls[1];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < PER; ++k)
+    if (wave + 4 * k < DVT) {
+      acc[0][k] = acc[0][k] * i1 - acc[1][k] * i2;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += acc[0][k][e] * acc[0][k][e];
+    }
+  ss = quad_sum(ss);
+  if (qd == 0) sss[wave][r] = ss;
+  __syncthreads();
+  ss = (sss[0][r] + sss[1][r]) + (sss[2][r] + sss[3][r]);
+  const float rn = out_scale * gate[(size_t)token * H + head] / sqrtf(ss / (float)Dv + eps);
+  if (valid) {
+    bf16_t* orow = out + ((size_t)token * H + head) * Dv + qd * 4;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int i = wave + 4 * k;
+      if (i < DVT) {
+        const u32x2_t o = {pack_bf2(acc[0][k][0] * rn, acc[0][k][1] * rn), pack_bf2(acc[0][k][2] * rn, acc[0][k][3] * rn)};
+        *reinterpret_cast<u32x2_t*>(orow + i * 16) = o;
+      }
+    }
+  }
 }
 
 }  // namespace
@@ -484,12 +514,15 @@ extern "C" int ssd_diffattn_store(const void* qkvg_rows, const void* q_norm_w, c
                                   int block_size, int f32, void* stream) {
   if (!qkvg_rows || !q_norm_w || !k_norm_w || !slots || !q_out || !gate_out || !k_cache || !v_cache) return SSD_ERR_ARG;
   if (T <= 0 || H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || block_size <= 0) return SSD_ERR_SHAPE;
+  int gy = (2 * H + 2 * G + 3) / 4;                 // one unit per wave when few tokens; fewer, fatter workgroups for prompt portions
+  if (T >= 64) gy = (gy + 7) / 8;
+  if (gy < 1) gy = 1;
   if (f32)
-    hipLaunchKernelGGL(diffattn_store_kernel<float>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)qkvg_rows,
+    hipLaunchKernelGGL(diffattn_store_kernel<float>, dim3(T, gy), dim3(256), 0, (hipStream_t)stream, (const float*)qkvg_rows,
                        (const float*)q_norm_w, (const float*)k_norm_w, eps, slots, (float*)q_out, (float*)gate_out, (float*)k_cache,
                        (float*)v_cache, H, G, D, Dv, block_size);
   else
-    hipLaunchKernelGGL(diffattn_store_kernel<bf16_t>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)qkvg_rows,
+    hipLaunchKernelGGL(diffattn_store_kernel<bf16_t>, dim3(T, gy), dim3(256), 0, (hipStream_t)stream, (const float*)qkvg_rows,
                        (const bf16_t*)q_norm_w, (const bf16_t*)k_norm_w, eps, slots, (bf16_t*)q_out, (float*)gate_out,
                        (bf16_t*)k_cache, (bf16_t*)v_cache, H, G, D, Dv, block_size);
   return LAUNCH_OK();
@@ -526,7 +559,7 @@ extern "C" int ssd_diffattn_paged(const void* q_rows, const void* k_cache, const
                        context_lens, cu_q, q_per_seq, B, H, G, D, Dv, block_size, scale, lambda, out_scale, eps, (bf16_t*)out_rows, split,
                        nsplit, (float*)workspace);
     if (nsplit > 1)
-      hipLaunchKernelGGL(diffattn_merge_kernel, dim3(B, G), dim3(64), 0, (hipStream_t)stream, (const float*)workspace, nsplit,
+      hipLaunchKernelGGL(diffattn_merge_kernel, dim3(B, G), dim3(256), 0, (hipStream_t)stream, (const float*)workspace, nsplit,
                          (const float*)gate, cu_q, q_per_seq, H, G, Dv, lambda, out_scale, eps, (bf16_t*)out_rows);
     return LAUNCH_OK();
   }

@@ -166,7 +166,7 @@ template <int NW>
 __global__ void __launch_bounds__(NW * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ y, int M, int N, int K, int epi,
                    const int* __restrict__ offsets, const int* __restrict__ row_idx, int idx_div) {
-  constexpr int U = 4;
+  constexpr int U = 8;
   __shared__ f32x4_t red[NW * 64];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, qd = lane >> 4;
   const int n0 = blockIdx.x * 16;

@@ -27,6 +27,19 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
   __syncthreads();
   return (red[0] + red[1]) + (red[2] + red[3]);
 }
+// the same for NT threads (a multiple of 256): waves summed in groups of four, the groups in order
+template <int NT>
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[wave] = v;
+  __syncthreads();
+  float s = 0.f;
+#pragma unroll
+  for (int q = 0; q < NT / 256; ++q) s += (red[4 * q] + red[4 * q + 1]) + (red[4 * q + 2] + red[4 * q + 3]);
+  return s;
+}
 
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -80,22 +93,22 @@ rmsnorm_add_res32_kernel(const float* __restrict__ y, const T* __restrict__ w, f
 //   x += w_post * rms(y);   then, if a next sublayer follows:  x += next_add (the re-injected embedding before a repeated pass),
 //   next_out = w_next * rms(x)  -- the input rows of the next sublayer's first GEMM.
 // Three launches (mix, post-norm + residual sum, next pre-norm) in one; the same arithmetic in the same order as the separate kernels.
-template <typename T>
-__global__ void __launch_bounds__(256)
+template <typename T, int NT>
+__global__ void __launch_bounds__(NT)
 sandwich_tail_kernel(const float* __restrict__ y, const float* __restrict__ ydn, const int32_t* __restrict__ inv,
                      const float* __restrict__ wt, const float* __restrict__ shared, int top, float* __restrict__ ytmp,
                      const T* __restrict__ w_post, float eps, float* __restrict__ x, const float* __restrict__ next_add,
                      const T* __restrict__ w_next, T* __restrict__ next_out, int W) {
-  __shared__ float red[4];
+  __shared__ float red[NT / 64];
   const int t = blockIdx.x;
   float* xr = x + (size_t)t * W;
   const float* yr = y ? y + (size_t)t * W : ytmp + (size_t)t * W;
   float ss = 0.f;
   if (y) {
-    for (int c = threadIdx.x; c < W; c += 256) { const float v = yr[c]; ss += v * v; }
+    for (int c = threadIdx.x; c < W; c += NT) { const float v = yr[c]; ss += v * v; }
   } else {
     float* yw = ytmp + (size_t)t * W;
-    for (int c = threadIdx.x; c < W; c += 256) {
+    for (int c = threadIdx.x; c < W; c += NT) {
       float v = 0.f;
       for (int j = 0; j < top; ++j) v = fmaf(wt[(size_t)t * top + j], ydn[(size_t)inv[(size_t)t * top + j] * W + c], v);
       if (shared) v += shared[(size_t)t * W + c];
@@ -103,19 +116,19 @@ sandwich_tail_kernel(const float* __restrict__ y, const float* __restrict__ ydn,
       ss += v * v;
     }
   }
-  ss = block_sum_256(ss, red);
+  ss = block_sum<NT>(ss, red);
   const float r = 1.0f / sqrtf(ss / (float)W + eps);
   float s2 = 0.f;
-  for (int c = threadIdx.x; c < W; c += 256) {
+  for (int c = threadIdx.x; c < W; c += NT) {
     float v = xr[c] + yr[c] * r * ldf<T>(w_post + c);
     if (next_add) v += next_add[(size_t)t * W + c];
     xr[c] = v;
     s2 += v * v;
   }
   if (!w_next) return;
-  s2 = block_sum_256(s2, red);
+  s2 = block_sum<NT>(s2, red);
   const float r2 = 1.0f / sqrtf(s2 / (float)W + eps);
-  for (int c = threadIdx.x; c < W; c += 256) stf<T>(next_out + (size_t)t * W + c, xr[c] * r2 * ldf<T>(w_next + c));
+  for (int c = threadIdx.x; c < W; c += NT) stf<T>(next_out + (size_t)t * W + c, xr[c] * r2 * ldf<T>(w_next + c));
 }
 
 __global__ void rows_f32_to_bf16_kernel(const float* __restrict__ src, bf16_t* __restrict__ dst, int cols, long ld_src, long ld_dst) {
@@ -182,12 +195,24 @@ extern "C" int ssd_sandwich_tail(const void* y_rows, const void* ydn_rows, const
   if (!y_rows && (!ydn_rows || !inv || !weights || !y_scratch || top <= 0)) return SSD_ERR_ARG;
   if ((next_weight == nullptr) != (next_out == nullptr) || (next_add && !next_weight)) return SSD_ERR_ARG;
   if (T <= 0 || W <= 0) return SSD_ERR_SHAPE;
+  if (T <= 64 && W >= 2048) {          // few rows: a row is a latency chain, so give it 1024 threads
+    if (f32)
+      hipLaunchKernelGGL((sandwich_tail_kernel<float, 1024>), dim3(T), dim3(1024), 0, (hipStream_t)stream, (const float*)y_rows,
+                         (const float*)ydn_rows, inv, weights, (const float*)shared_rows, top, (float*)y_scratch,
+                         (const float*)post_weight, eps, (float*)x, (const float*)next_add, (const float*)next_weight, (float*)next_out, W);
+    else
+      hipLaunchKernelGGL((sandwich_tail_kernel<bf16_t, 1024>), dim3(T), dim3(1024), 0, (hipStream_t)stream, (const float*)y_rows,
+                         (const float*)ydn_rows, inv, weights, (const float*)shared_rows, top, (float*)y_scratch,
+                         (const bf16_t*)post_weight, eps, (float*)x, (const float*)next_add, (const bf16_t*)next_weight,
+                         (bf16_t*)next_out, W);
+    return LAUNCH_OK();
+  }
   if (f32)
-    hipLaunchKernelGGL(sandwich_tail_kernel<float>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)y_rows,
+    hipLaunchKernelGGL((sandwich_tail_kernel<float, 256>), dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)y_rows,
                        (const float*)ydn_rows, inv, weights, (const float*)shared_rows, top, (float*)y_scratch,
                        (const float*)post_weight, eps, (float*)x, (const float*)next_add, (const float*)next_weight, (float*)next_out, W);
   else
-    hipLaunchKernelGGL(sandwich_tail_kernel<bf16_t>, dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)y_rows,
+    hipLaunchKernelGGL((sandwich_tail_kernel<bf16_t, 256>), dim3(T), dim3(256), 0, (hipStream_t)stream, (const float*)y_rows,
                        (const float*)ydn_rows, inv, weights, (const float*)shared_rows, top, (float*)y_scratch,
                        (const bf16_t*)post_weight, eps, (float*)x, (const float*)next_add, (const bf16_t*)next_weight,
                        (bf16_t*)next_out, W);

@@ -259,10 +259,11 @@ def test_diffattn_decode_rows_of_several_sequences(f32, Hh, G, D, Dv, bs):
 
 @pytest.mark.parametrize("f32", MODES)
 @pytest.mark.parametrize("routed", [False, True])
-def test_sandwich_tail_equals_its_separate_launches(f32, routed):
+@pytest.mark.parametrize("W", [200, 2048])          # 2048: few rows of a wide model take the 1024-thread form (another summation order)
+def test_sandwich_tail_equals_its_separate_launches(f32, routed, W):
     from ssd_amd.hip import ops as H
     g = torch.Generator().manual_seed(11)
-    T, W, top, eps = 7, 200, 3, 1e-5
+    T, top, eps = 7, 3, 1e-5
     el = _elem(f32)
     wp, wn = _rand((W,), f32, g) + 1, _rand((W,), f32, g) + 1
     x0 = torch.randn(T, W, generator=g).to(DEV)
@@ -284,10 +285,10 @@ def test_sandwich_tail_equals_its_separate_launches(f32, routed):
     xb, nb, scratch = x0.clone(), torch.zeros(T, W, dtype=el, device=DEV), torch.zeros(T, W, device=DEV)
     src = dict(ydn=ydn, inv=inv, weights=wt, shared=sh, top=top, y_scratch=scratch) if routed else dict(y=y)
     H.sandwich_tail(wp, eps, xb, T, W, f32, next_add=add, next_weight=wn, next_out=nb, **src)
-    torch.testing.assert_close(xb, xa, rtol=1e-6, atol=1e-6)
-    torch.testing.assert_close(nb.float(), na.float(), **(dict(rtol=1e-6, atol=1e-6) if f32 else dict(rtol=1e-2, atol=1e-2)))
+    torch.testing.assert_close(xb, xa, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(nb.float(), na.float(), **(dict(rtol=1e-5, atol=1e-5) if f32 else dict(rtol=1e-2, atol=1e-2)))
     xc = x0.clone()                     # the last sublayer of a model: no next norm
     H.sandwich_tail(wp, eps, xc, T, W, f32, **src)
     xd = x0.clone()
     H.rmsnorm_add_res32(y, wp, eps, xd, T, W, f32)
-    torch.testing.assert_close(xc, xd, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(xc, xd, rtol=1e-5, atol=1e-5)

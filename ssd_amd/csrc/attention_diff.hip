@@ -305,21 +305,40 @@ diffattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc
     const int k0 = st << 5;
     const size_t pg = (size_t)table[k0 / bs] * G + g;
     const int koff = k0 % bs;
+    // every load of the step is issued before the first product: one memory round trip per 32 keys (the value tiles do not wait for
+    // the softmax)
+    u32x4_t kreg[2][2][DM_KS];
+    u32x2_t vlo[DM_DVT], vhi[DM_DVT];
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+      for (int hg = 0; hg < 2; ++hg) {
+        const bf16_t* kr = kc + (pg * bs + koff + hg * 16 + r) * 2 * D + m * D + qd * 8;
+#pragma unroll
+        for (int ks = 0; ks < DM_KS; ++ks) {
+          kreg[m][hg][ks] = u32x4_t{0u, 0u, 0u, 0u};
+          if (ks < KS && ks * 32 + qd * 8 < D) kreg[m][hg][ks] = *reinterpret_cast<const u32x4_t*>(kr + ks * 32);
+        }
+      }
+#pragma unroll
+    for (int i = 0; i < DM_DVT; ++i) {
+      vlo[i] = u32x2_t{0u, 0u};
+      vhi[i] = u32x2_t{0u, 0u};
+      if (i < DVT) {
+        const bf16_t* vp = vt + (pg * Dv + i * 16 + r) * bs + koff + qd * 4;
+        vlo[i] = *reinterpret_cast<const u32x2_t*>(vp);
+        vhi[i] = *reinterpret_cast<const u32x2_t*>(vp + 16);
+      }
+    }
     f32x4_t s[2][2];
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
       for (int hg = 0; hg < 2; ++hg) {
         s[m][hg] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-        const bf16_t* kr = kc + (pg * bs + koff + hg * 16 + r) * 2 * D + m * D + qd * 8;
 #pragma unroll
-        for (int ks = 0; ks < DM_KS; ++ks) {
-          if (ks < KS) {
-            u32x4_t a = {0u, 0u, 0u, 0u};
-            if (ks * 32 + qd * 8 < D) a = *reinterpret_cast<const u32x4_t*>(kr + ks * 32);
-            s[m][hg] = mfma16(a, qreg[m][ks], s[m][hg]);
-          }
-        }
+        for (int ks = 0; ks < DM_KS; ++ks)
+          if (ks < KS) s[m][hg] = mfma16(kreg[m][hg][ks], qreg[m][ks], s[m][hg]);
       }
     u32x4_t pb[2];
 #pragma unroll
@@ -353,9 +372,7 @@ diffattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc
 #pragma unroll
     for (int i = 0; i < DM_DVT; ++i) {
       if (i < DVT) {
-        const bf16_t* vp = vt + (pg * Dv + i * 16 + r) * bs + koff + qd * 4;
-        u32x2_t lo = *reinterpret_cast<const u32x2_t*>(vp);
-        u32x2_t hi = *reinterpret_cast<const u32x2_t*>(vp + 16);
+        u32x2_t lo = vlo[i], hi = vhi[i];
         if (tail) {         // keys past the sequence: whatever the page holds there must not meet a zero weight as NaN
           const int kb = k0 + qd * 4;
           if (kb + 0 >= ctx) lo.x &= 0xffff0000u;

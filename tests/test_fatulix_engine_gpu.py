@@ -47,6 +47,9 @@ CONFIGS = {
     "loop_inside": dict(n_layers=4, loop=(1, 3, 3), no_mlp_layers=(2,), heads=4, kv_heads=2, dim=16, vdim=24, width=64, vocab=96),
     "mha_top1_noshared": dict(n_layers=2, loop=(0, 0, 1), heads=3, kv_heads=3, dim=20, vdim=12, width=72, vocab=50, experts=3, top=1,
                               shared_ff=0, ff=40),
+    # head sizes the MFMA attention takes (dim % 8, vdim % 16) -- with 32-token pages the bf16 runs use it, tile and key-split forms
+    "mfma_sizes": dict(n_layers=3, loop=(1, 2, 2), heads=4, kv_heads=2, dim=24, vdim=32, width=96, vocab=80, experts=4, top=2, ff=32,
+                       shared_ff=64),
     "mqa_all_experts": dict(n_layers=2, loop=(0, 2, 2), heads=6, kv_heads=1, dim=40, vdim=72, width=100, vocab=131, experts=3, top=3,
                             ff=24, shared_ff=56, diff=0.45, scale=0.3),
 }
@@ -54,6 +57,8 @@ CONFIGS = {
 
 def make(name, seed=0):
     cfg = F.make_config(**CONFIGS[name])
+    if name == "mfma_sizes":
+        cfg["layers"][2]["mixer"].update(heads=8, kv_heads=1, dim=8, vdim=16, scale=0.5)        # 8 rows per token: prompt portions of 3+ tokens leave the key-split form
     if name == "loop_inside":       # layers of one model may differ in every size
         cfg["layers"][3]["mixer"].update(heads=2, kv_heads=1, dim=24, vdim=40, diff=0.1, scale=0.2)
         cfg["layers"][3]["mlp"]["router"].update(experts=5, top=3)
@@ -198,3 +203,29 @@ def test_greedy_generation_through_llm_generate(tmp_path, dtype):
         assert ((top - chosen) <= margin * lg.std()).all(), (top - chosen).max()
         if dtype == "float32":
             assert gen == lg.argmax(-1).tolist()
+
+
+@pytest.mark.parametrize("block_size", [32, 64])
+def test_bf16_mfma_attention_through_the_engine_portions_decoding_and_mixed_steps(tmp_path, block_size):
+    """bf16 with 32 / 64-token pages and aligned head sizes: prompt portions run the MFMA tile form, decoded tokens (and short portions)
+    the key-split form; cuts at and next to page borders; two requests share steps; every position against the oracle."""
+    cfg, w = make("mfma_sizes", seed=9)
+    n = 150
+    ta, tb = tokens(n, cfg["vocab"], 30), tokens(77, cfg["vocab"], 31)
+    ra, rb = F.forward(cfg, w, ta, torch.float64), F.forward(cfg, w, tb, torch.float64)
+    eng = engine(tmp_path, cfg, w, "bfloat16", max_tokens=320, block_size=block_size)
+    whole = _replay(eng, "w", ta, [n])
+    assert close(whole, ra, "bfloat16"), rel_err(whole, ra)
+    cuts = [block_size - 1, block_size, block_size + 1, 2 * block_size + 2, 100] + list(range(101, n + 1))
+    got = _replay(eng, "c", ta, cuts)
+    assert close(got, ra, "bfloat16"), rel_err(got, ra)
+    assert rel_err(got, whole) < 0.05          # the same bf16 inputs, other fp32 summation orders only
+    # two requests, portions of one beside single tokens of the other, pages of the finished requests above in use again
+    ga, gb, ia, ib = [], [], 0, 0
+    plan = [(70, 1), (1, 40), (1, 1), (30, 1), (1, 33), (47, 1)]
+    for ca, cb in plan:
+        lg = eng.step([{"id": "a", "tokens": ta[ia:ia + ca], "want": list(range(ca))}, {"id": "b", "tokens": tb[ib:ib + cb], "want": list(range(cb))}],
+                      [x for x, done in (("a", ia + ca == n), ("b", ib + cb == 77)) if done])
+        ga.append(lg[:ca]); gb.append(lg[ca:]); ia += ca; ib += cb
+    assert ia == n and ib == 77
+    assert close(torch.cat(ga), ra, "bfloat16") and close(torch.cat(gb), rb, "bfloat16")

@@ -394,7 +394,7 @@ diffattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc
   if (split) {
     // ---- merge the four waves' partials in wave order ----
     float* sm = smem;                       // [4 waves][2 maps][2: max, sum][16 rows]
-    float* sbuf = smem + 4 * 2 * 2 * 16;    // [2 maps][DVT][64 lanes][4]
+    float* sbuf = smem + 4 * 2 * 2 * 16;    // [3 waves][2 maps][DVT][64 lanes][4]
     if (qd == 0) {
 #pragma unroll
       for (int m = 0; m < 2; ++m) { sm[((wave * 2 + m) * 2 + 0) * 16 + r] = mx[m]; sm[((wave * 2 + m) * 2 + 1) * 16 + r] = ls[m]; }
@@ -415,23 +415,23 @@ diffattn_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc
       ls[m] = L;
       mx[m] = M;
     }
-    for (int w = 1; w < 4; ++w) {
-      if (wave == w) {
+    // waves 1..3 leave their (already rescaled) O fragments in areas of their own; wave 0 adds them in wave order: one barrier
+    const size_t area = (size_t)2 * DVT * 64 * 4;
+    if (wave > 0) {
+#pragma unroll
+      for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int i = 0; i < DM_DVT; ++i)
+          if (i < DVT) *reinterpret_cast<f32x4_t*>(sbuf + (wave - 1) * area + ((size_t)(m * DVT + i) * 64 + lane) * 4) = acc[m][i];
+    }
+    __syncthreads();
+    if (wave == 0) {
+      for (int w = 0; w < 3; ++w)
 #pragma unroll
         for (int m = 0; m < 2; ++m)
 #pragma unroll
           for (int i = 0; i < DM_DVT; ++i)
-            if (i < DVT) *reinterpret_cast<f32x4_t*>(sbuf + ((size_t)(m * DVT + i) * 64 + lane) * 4) = acc[m][i];
-      }
-      __syncthreads();
-      if (wave == 0) {
-#pragma unroll
-        for (int m = 0; m < 2; ++m)
-#pragma unroll
-          for (int i = 0; i < DM_DVT; ++i)
-            if (i < DVT) acc[m][i] += *reinterpret_cast<const f32x4_t*>(sbuf + ((size_t)(m * DVT + i) * 64 + lane) * 4);
-      }
-      __syncthreads();
+            if (i < DVT) acc[m][i] += *reinterpret_cast<const f32x4_t*>(sbuf + w * area + ((size_t)(m * DVT + i) * 64 + lane) * 4);
     }
     if (wave != 0) return;
   }
@@ -559,7 +559,7 @@ extern "C" int ssd_diffattn_paged(const void* q_rows, const void* k_cache, const
     const int R = H / G;
     const int split = max_q * R <= 16 ? 1 : 0;
     const int gx = split ? B : ((long)T * R + 63) / 64 + B;
-    const size_t lds_m = split ? (size_t)(4 * 2 * 2 * 16 + 2 * (Dv / 16) * 64 * 4) * 4 : 0;
+    const size_t lds_m = split ? (size_t)(4 * 2 * 2 * 16 + 3 * 2 * (Dv / 16) * 64 * 4) * 4 : 0;
     // decoding rows of few sequences: cut the keys over more workgroups (a launch of B * G workgroups leaves most of the chip idle)
     // when the caller gave a workspace and says the contexts are long; every wave keeps at least 4 steps of 32 keys
     int nsplit = 1;

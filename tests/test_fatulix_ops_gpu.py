@@ -152,7 +152,7 @@ def _paged_ref(qo, kc, vt, gate, bt, pos, seq, Hh, G, D, Dv, bs, scale, lam, osc
     return out
 
 
-SHAPES = [(4, 2, 56, 80, 64), (8, 2, 64, 128, 32), (4, 4, 128, 64, 64), (5, 5, 8, 16, 32),          # the MFMA form takes these in bf16
+SHAPES = [(4, 2, 56, 80, 64), (8, 2, 64, 128, 32), (4, 4, 128, 64, 64), (5, 5, 8, 16, 32), (6, 2, 16, 32, 32),   # the MFMA form takes these in bf16
           (3, 3, 20, 24, 16), (6, 1, 64, 40, 32), (2, 2, 136, 512 - 8, 64)]                          # scalar form only
 
 
@@ -207,7 +207,7 @@ def test_diffattn_store_and_paged_over_scattered_pages(f32, Hh, G, D, Dv, bs):
 
 
 @pytest.mark.parametrize("f32", MODES)
-@pytest.mark.parametrize("Hh,G,D,Dv,bs", SHAPES[:5])
+@pytest.mark.parametrize("Hh,G,D,Dv,bs", SHAPES[:6])
 def test_diffattn_decode_rows_of_several_sequences(f32, Hh, G, D, Dv, bs):
     """A batch of sequences with different lengths bringing one or two rows each (decoding, the last tokens of a portion): keys just
     inside the visible range count, the key after a row's position does not (the second row's key is in the cache when the first row

@@ -107,3 +107,19 @@ def test_trace_engine_takes_and_returns_pages():
         eng.step([{"id": "d", "tokens": [5], "want": []}])                          # no page left
     eng.step([], end=["b", "c"])
     assert len(eng.blocks.free_block_ids) == 4 and not eng.live
+
+
+def test_bench_option_and_equal_size_pairs():
+    """bench.py accepts --workload fatulix next to its default; every benchmarked size pairs a Fatulix model with a Llama decoder of the
+    same width, projection sizes and feed-forward parameters per token."""
+    import bench
+    from ssd_amd.utils import arch_bench
+    assert bench.parse([]).workload == "c4"                                  # the default workload is untouched
+    a = bench.parse(["--workload", "fatulix", "--arch-size", "w2048", "--arch-batch", "1"])
+    assert a.workload == "fatulix" and a.arch_size == "w2048" and a.arch_batch == 1
+    for size in arch_bench.SIZES:
+        fat, llama = arch_bench.models(size)
+        m, ml = fat.layers[0].mixer, fat.layers[0].mlp
+        assert fat.hidden_size == llama.hidden_size and fat.vocab_size == llama.vocab_size and len(fat.layers) == llama.num_layers
+        assert m.heads * 2 * m.dim == llama.q_size and m.kv_heads * 2 * m.dim == llama.kv_size == m.kv_heads * m.vdim
+        assert ml.top * 2 * ml.ff + 2 * ml.shared_ff == 3 * llama.intermediate_size

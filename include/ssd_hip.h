@@ -31,7 +31,7 @@ extern "C" {
 
 /* Bumped whenever a signature or a semantic of this header changes; ssd_abi_version() returns the value the library was built
  * with, so a consumer compiled against another header can tell (tests/abi_consumer.c does). */
-#define SSD_HIP_ABI_VERSION 3
+#define SSD_HIP_ABI_VERSION 4
 
 #define SSD_OK 0
 #define SSD_ERR_SHAPE (-1)
@@ -425,6 +425,61 @@ int ssd_moe_route(const float* logits, int32_t* idx, float* weights, int T, int 
 int ssd_moe_plan(const int32_t* idx, int T, int top, int E, int32_t* offsets, int32_t* perm, int32_t* inv, void* stream);
 int ssd_moe_combine(const void* y_rows, const int32_t* inv, const float* weights, const void* shared_rows, void* out_rows, int T,
                     int top, int W, void* stream);
+
+/* G products in one launch (per-head matrices over column slices of token-major rows): group g multiplies x_rows + g * gsx (row
+ * stride ldx) by w_rows + g * N * K and writes y + g * gsy (row stride ldy; strides in elements of the respective type). */
+int ssd_gemm_rows_batched(const void* x_rows, const void* w_rows, void* y, int M, int N, int K, int G, long ldx, long gsx, long ldy,
+                          long gsy, int epilogue, int f32, void* stream);
+
+/* Parallel layers with Dynamic-Tanh norms, dyt(x) = tanh(alpha * x) * weight + bias (csrc/dyt.hip); alpha: one fp32 number in
+ * device memory.  ssd_dyt_embed: x (fp32 [T][W]) = dyt(table[ids]); x0 (optional) a second fp32 copy; cat (optional) an element-type
+ * copy with row stride ld_cat.  ssd_dyt_rows: out[r] = dyt(x[i]), i = gather[r] or r; add_vec (optional, [W], no gather): x += add_vec
+ * first, written back. */
+int ssd_dyt_embed(const int64_t* ids, const void* table, const float* alpha, const void* weight, const void* bias, void* x, void* x0,
+                  void* cat, long ld_cat, int T, int W, long vocab, int f32, void* stream);
+int ssd_dyt_rows(void* x, const void* add_vec, const float* alpha, const void* weight, const void* bias, void* out_rows,
+                 const int32_t* gather, int T, int W, int f32, void* stream);
+/* x += y_mix + ff: ff = y_ff (fp32 [T][W]) or, when y_ff is NULL and ydn_rows is given, sum_j weights[t][j] * ydn_rows[inv[t*top+j]]
+ * (+ sigmoid(shared_gate[t * ld_shared_gate]) * shared_rows[t]; a NULL shared_gate means 1), or 0.  Then next_out = dyt(x) with
+ * next_alpha / next_weight / next_bias (optional) and cat = x as element-type rows of stride ld_cat (optional). */
+int ssd_parallel_tail(void* x, const void* y_mix, const void* y_ff, const void* ydn_rows, const int32_t* inv, const float* weights,
+                      int top, const void* shared_rows, const float* shared_gate, long ld_shared_gate, const float* next_alpha,
+                      const void* next_weight, const void* next_bias, void* next_out, void* cat, long ld_cat, int T, int W, int f32,
+                      void* stream);
+/* out[r][c] = act(ab[r][c]) * ab[r][F + c] for fp32 rows [rows][2F]; act 0: silu, 1: tanh-form gelu. */
+int ssd_glu_rows(const void* ab_rows, void* out_rows, int rows, int F, int act, int f32, void* stream);
+
+/* Latent attention with a sliding window (csrc/attention_latent.hip).  proj_rows fp32 [T][ld] = [dq (q_rank) | latent (kv_rank) |
+ * rotated key part (rot) | gate logits (H)].  Store: cq_out [T][q_rank] = rms(dq) * q_norm_w; cache row slots[t] (-1: none) of
+ * cache [rows][kv_rank + rot] = [rms(latent) * kv_norm_w | rope(rotated key part)]; gate_out fp32 [T][H] = sigmoid.  rope turns the
+ * first rot_dims entries (entry i pairs with i + rot_dims / 2) by positions[t] * freqs[i] with cos and sin times mag. */
+int ssd_latent_store(const void* proj_rows, long ld, int q_rank, int kv_rank, int rot, int H, const void* q_norm_w,
+                     const void* kv_norm_w, float eps, const int64_t* positions, const float* freqs, float mag, int rot_dims,
+                     const int32_t* slots, void* cq_out, void* cache, void* gate_out, int T, int f32, void* stream);
+/* out[t][h] (kv_rank wide) = gate[t][h] * sum_j softmax_j(scale * (<q_abs[t][h], c_j> + <rope(q_rows[t][h][D:]), k_j>)) c_j over the
+ * keys j of the token's sequence with 0 <= positions[t] - j < window (window <= 0: all keys up to the token); q_abs fp32
+ * [T][H][kv_rank], q_rows [T][H][D + rot].  Sequences: cu_q int32 [B+1] row ranges, or q_per_seq rows each when cu_q is NULL. */
+int ssd_latent_attn(const void* q_abs, const void* q_rows, const void* cache, const void* gate, const int32_t* block_tables,
+                    int max_blocks, const int64_t* positions, const int32_t* cu_q, int q_per_seq, int B, int T, int H, int D, int rot,
+                    int kv_rank, int block_size, int window, float scale, const float* freqs, float mag, int rot_dims, void* out_rows,
+                    int f32, void* stream);
+
+/* Linear attention with per-head decay over a recurrent fp32 state (csrc/lightning.hip).  proj_rows fp32 [T][ld] holds q at q_off
+ * ([H][D]), k at k_off ([H][D]), v at v_off ([H][Dv]), each passed through silu.  Per sequence b (rows cu_q[b] .. cu_q[b+1]-1, or
+ * q_per_seq rows each) and head: S = state[state_slots[b]][h] (zero when the first row's position is 0), per row S = decay[h] * S +
+ * k v^T, out = S^T q (fp32 [T][H*Dv]); S is written back. */
+int ssd_lightning_scan(const void* proj_rows, long ld, int q_off, int k_off, int v_off, const float* decay, const int64_t* positions,
+                       const int32_t* cu_q, int q_per_seq, const int32_t* state_slots, void* state, void* out_rows, int B, int H, int D,
+                       int Dv, void* stream);
+/* out[t] = weight * o[t] / sqrt(mean(o[t]^2) + eps) * sigmoid(proj_rows[t][g_off ..]) over N = H * Dv entries, element-type rows. */
+int ssd_lightning_gate_norm(const void* o_rows, const void* proj_rows, long ld, int g_off, const void* weight, float eps,
+                            void* out_rows, int T, int N, int f32, void* stream);
+
+/* Router of the softmax-then-choose kind: scores = softmax(logits[t][0..E)) (row stride ld), experts in `groups` contiguous groups of
+ * which the `keep` with the largest best score stay eligible, the `top` largest eligible scores -> idx, weights = score / (sum of
+ * the chosen + 1e-20) * scale. */
+int ssd_moe_route_softmax(const float* logits, long ld, int32_t* idx, float* weights, int T, int E, int top, int groups, int keep,
+                          float scale, void* stream);
 
 /* hipGraph capture for a host that is not PyTorch -- the reference captures its decode / verify / glue / tree steps with
  * torch.cuda.CUDAGraph (ssd/engine/helpers/cudagraph_helpers.py:20-120); every entry point above only enqueues on `stream`, so the calls

@@ -100,6 +100,8 @@ class Config:
         self.max_model_len = min(self.max_model_len, self.hf_config.max_position_embeddings)
         if self.speculate:
             assert self.draft is not None, "speculate=True needs a draft model"
+            assert not getattr(self.hf_config, "recurrent", False), \
+                "speculation rolls rejected tokens back by position; a recurrent state cannot be rolled back"
             if self.draft_hf_config is None:
                 self.draft_hf_config = resolve_model_config(self.draft)
             self.max_model_len = min(self.max_model_len, self.draft_hf_config.max_position_embeddings)

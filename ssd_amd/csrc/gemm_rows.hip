@@ -9,6 +9,8 @@
 //   grouped: offsets[E+1] cuts the (sorted) rows into E runs, run e multiplies by w + e * N * K; row_idx (optional) names the x row
 //   of every sorted row as row_idx[r] / idx_div; tiles never straddle two runs (blockIdx.y walks a list of at most
 //   ceil(rows / 64) + E tiles, found by a scan of offsets).
+//   batched: G independent products in one launch (blockIdx.z / blockIdx.y = g): x + g * gsx with row stride ldx, w + g * N * K,
+//   y + g * gsy with row stride ldy -- per-head products whose operands are column slices of token-major rows.
 #include "common.h"
 
 namespace {
@@ -55,25 +57,28 @@ __device__ __forceinline__ void stage_tile(T* lds, const T* __restrict__ src, co
 
 // epilogue 0: fp32 rows; 1: relu(v)^2 as element-type rows; 2: element-type rows
 template <typename T>
-__device__ __forceinline__ void store_out(void* y, long row, int N, int n, float v, int epi) {
+__device__ __forceinline__ void store_out(void* y, long row, long ldy, long n, float v, int epi) {
   if (epi == 0) {
-    reinterpret_cast<float*>(y)[row * N + n] = v;
+    reinterpret_cast<float*>(y)[row * ldy + n] = v;
   } else {
     if (epi == 1) { v = v > 0.f ? v : 0.f; v = v * v; }
-    Elem<T>::st(reinterpret_cast<T*>(y) + row * N + n, v);
+    Elem<T>::st(reinterpret_cast<T*>(y) + row * ldy + n, v);
   }
 }
 
 template <typename T>
 __global__ void __launch_bounds__(256)
 gemm_rows_kernel(const T* __restrict__ x, const T* __restrict__ w, void* __restrict__ y, int M, int N, int K, int epi,
-                 const int* __restrict__ offsets, int E, const int* __restrict__ row_idx, int idx_div, bool vec_ok) {
+                 const int* __restrict__ offsets, int E, const int* __restrict__ row_idx, int idx_div, bool vec_ok, long ldx, long ldy,
+                 long gsx, long gsy) {
   constexpr int PAD = 16 / sizeof(T);
   constexpr int LDT = BK + PAD;
   __shared__ __attribute__((aligned(16))) T sx[BM * LDT];
   __shared__ __attribute__((aligned(16))) T sw[BN * LDT];
   int row0 = blockIdx.y * BM, row_end = M;
-  const T* wg = w;
+  const T* wg = w + (size_t)blockIdx.z * N * K;
+  x += (size_t)blockIdx.z * gsx;
+  const long ycol = (long)blockIdx.z * gsy;
   if (offsets) {           // grouped: find the run and the tile inside it that this workgroup owns
     int tile = blockIdx.y, e = 0;
     for (; e < E; ++e) {
@@ -95,7 +100,7 @@ gemm_rows_kernel(const T* __restrict__ x, const T* __restrict__ w, void* __restr
 #pragma unroll
     for (int i = 0; i < 4; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     for (int k0 = 0; k0 < K; k0 += BK) {
-      stage_tile<T, LDT>(sx, x, row_idx, idx_div, row0, row_end, k0, K, K, vec_ok);
+      stage_tile<T, LDT>(sx, x, row_idx, idx_div, row0, row_end, k0, K, ldx, vec_ok);
       stage_tile<T, LDT>(sw, wg, nullptr, 1, n0, N, k0, K, K, vec_ok);
       __syncthreads();
       const u32x4_t b = *reinterpret_cast<const u32x4_t*>(sx + (wave * 16 + (lane & 15)) * LDT + (lane >> 4) * 8);
@@ -113,7 +118,7 @@ gemm_rows_kernel(const T* __restrict__ x, const T* __restrict__ w, void* __restr
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int n = n0 + nt * 16 + (lane >> 4) * 4 + r;
-          if (n < N) store_out<T>(y, m, N, n, acc[nt][r], epi);
+          if (n < N) store_out<T>(y, m, ldy, ycol + n, acc[nt][r], epi);
         }
     }
   } else {
@@ -125,7 +130,7 @@ gemm_rows_kernel(const T* __restrict__ x, const T* __restrict__ w, void* __restr
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
     for (int k0 = 0; k0 < K; k0 += BK) {
-      stage_tile<T, LDT>(sx, x, row_idx, idx_div, row0, row_end, k0, K, K, vec_ok);
+      stage_tile<T, LDT>(sx, x, row_idx, idx_div, row0, row_end, k0, K, ldx, vec_ok);
       stage_tile<T, LDT>(sw, wg, nullptr, 1, n0, N, k0, K, K, vec_ok);
       __syncthreads();
 #pragma unroll 8
@@ -149,7 +154,7 @@ gemm_rows_kernel(const T* __restrict__ x, const T* __restrict__ w, void* __restr
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int n = n0 + tn + 16 * j;
-        if (n < N) store_out<T>(y, m, N, n, acc[i][j], epi);
+        if (n < N) store_out<T>(y, m, ldy, ycol + n, acc[i][j], epi);
       }
     }
   }
@@ -165,13 +170,20 @@ gemm_rows_kernel(const T* __restrict__ x, const T* __restrict__ w, void* __restr
 template <int NW>
 __global__ void __launch_bounds__(NW * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ y, int M, int N, int K, int epi,
-                   const int* __restrict__ offsets, const int* __restrict__ row_idx, int idx_div) {
+                   const int* __restrict__ offsets, const int* __restrict__ row_idx, int idx_div, long ldx, long ldy, long gsx,
+                   long gsy) {
   constexpr int U = 8;
   __shared__ f32x4_t red[NW * 64];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, qd = lane >> 4;
   const int n0 = blockIdx.x * 16;
   int m_begin = 0, m_end = M;
   const bf16_t* wg = w;
+  long ycol = 0;
+  if (!offsets) {          // batched (or a single product: blockIdx.y == 0)
+    wg = w + (size_t)blockIdx.y * N * K;
+    x += (size_t)blockIdx.y * gsx;
+    ycol = (long)blockIdx.y * gsy;
+  }
   if (offsets) {
     m_begin = offsets[blockIdx.y];
     m_end = offsets[blockIdx.y + 1];
@@ -185,7 +197,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, v
     const int mrow = m0 + r;
     const bool mvalid = mrow < m_end;
     const long xrow = mvalid ? (row_idx ? (long)(row_idx[mrow] / idx_div) : (long)mrow) : 0;
-    const bf16_t* xp = x + xrow * K + qd * 8;
+    const bf16_t* xp = x + xrow * ldx + qd * 8;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
     for (int kt0 = wave * U; kt0 < KT; kt0 += NW * U) {
       u32x4_t a[U], b[U];
@@ -211,7 +223,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, v
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int n = n0 + qd * 4 + e;
-          if (n < N) store_out<bf16_t>(y, mrow, N, n, sum[e], epi);
+          if (n < N) store_out<bf16_t>(y, mrow, ldy, ycol + n, sum[e], epi);
         }
       }
     }
@@ -222,39 +234,45 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, v
 constexpr int SKINNY_MAX_ROWS = 16, SKINNY_MAX_GROUPED_ROWS = 64;
 
 int launch(const void* x, const void* w, void* y, int M, int N, int K, int epi, const int* offsets, int E, const int* row_idx,
-           int idx_div, int f32, void* stream) {
+           int idx_div, int f32, void* stream, int G = 1, long ldx = 0, long gsx = 0, long ldy = 0, long gsy = 0) {
   if (!x || !w || !y) return SSD_ERR_ARG;
   if (M <= 0 || N <= 0 || K <= 0 || epi < 0 || epi > 2) return SSD_ERR_SHAPE;
   if (offsets && E <= 0) return SSD_ERR_SHAPE;
-  if (!f32 && K % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 &&
+  if (G < 1 || G > 65535 || (G > 1 && offsets)) return SSD_ERR_SHAPE;
+  if (ldx == 0) ldx = K;
+  if (ldy == 0) ldy = N;
+  if (ldx < K || ldy < N) return SSD_ERR_SHAPE;
+  const int esz0 = f32 ? 4 : 2;
+  const bool x_vec = ((size_t)ldx * esz0) % 16 == 0 && ((size_t)gsx * esz0) % 16 == 0 && (uintptr_t)x % 16 == 0;
+  if (!f32 && K % 8 == 0 && x_vec && (uintptr_t)w % 16 == 0 &&
       M <= (offsets ? SKINNY_MAX_GROUPED_ROWS : SKINNY_MAX_ROWS)) {
     const int groups = (N + 15) / 16;
-    const dim3 sg(groups, offsets ? E : 1);
+    const dim3 sg(groups, offsets ? E : G);
     const int id = idx_div < 1 ? 1 : idx_div;
-    const long wgs = (long)groups * (offsets ? (M < E ? M : E) : 1);          // workgroups that have rows
+    const long wgs = (long)groups * (offsets ? (M < E ? M : E) : G);          // workgroups that have rows
     // few workgroups: more waves each (a CU pulls from HBM what its waves have in flight), as long as every wave gets k-tiles
     const int kt = (K + 31) / 32;
     if (wgs < 256 && kt >= 64)
       hipLaunchKernelGGL(gemm_skinny_kernel<16>, sg, dim3(1024), 0, (hipStream_t)stream, (const bf16_t*)x, (const bf16_t*)w, y, M, N, K,
-                         epi, offsets, row_idx, id);
+                         epi, offsets, row_idx, id, ldx, ldy, gsx, gsy);
     else if (wgs < 1024 && kt >= 32)
       hipLaunchKernelGGL(gemm_skinny_kernel<8>, sg, dim3(512), 0, (hipStream_t)stream, (const bf16_t*)x, (const bf16_t*)w, y, M, N, K,
-                         epi, offsets, row_idx, id);
+                         epi, offsets, row_idx, id, ldx, ldy, gsx, gsy);
     else
       hipLaunchKernelGGL(gemm_skinny_kernel<4>, sg, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x, (const bf16_t*)w, y, M, N, K,
-                         epi, offsets, row_idx, id);
+                         epi, offsets, row_idx, id, ldx, ldy, gsx, gsy);
     return hipGetLastError() == hipSuccess ? SSD_OK : SSD_ERR_LAUNCH;
   }
   const int tiles_m = (M + BM - 1) / BM + (offsets ? E : 0);
-  const dim3 grid((N + BN - 1) / BN, tiles_m);
+  const dim3 grid((N + BN - 1) / BN, tiles_m, G);
   const int esz = f32 ? 4 : 2;
-  const bool vec_ok = ((size_t)K * esz) % 16 == 0 && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
+  const bool vec_ok = ((size_t)K * esz) % 16 == 0 && x_vec && ((uintptr_t)w % 16 == 0);
   if (f32)
     hipLaunchKernelGGL(gemm_rows_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)x, (const float*)w, y, M, N, K,
-                       epi, offsets, E, row_idx, idx_div < 1 ? 1 : idx_div, vec_ok);
+                       epi, offsets, E, row_idx, idx_div < 1 ? 1 : idx_div, vec_ok, ldx, ldy, gsx, gsy);
   else
     hipLaunchKernelGGL(gemm_rows_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x, (const bf16_t*)w, y, M, N,
-                       K, epi, offsets, E, row_idx, idx_div < 1 ? 1 : idx_div, vec_ok);
+                       K, epi, offsets, E, row_idx, idx_div < 1 ? 1 : idx_div, vec_ok, ldx, ldy, gsx, gsy);
   return hipGetLastError() == hipSuccess ? SSD_OK : SSD_ERR_LAUNCH;
 }
 
@@ -270,4 +288,10 @@ extern "C" int ssd_gemm_rows_grouped(const void* x_rows, const void* w_rows, voi
                                      void* stream) {
   if (!offsets) return SSD_ERR_ARG;
   return launch(x_rows, w_rows, y, rows, N, K, epilogue, offsets, E, row_idx, idx_div, f32, stream);
+}
+
+extern "C" int ssd_gemm_rows_batched(const void* x_rows, const void* w_rows, void* y, int M, int N, int K, int G, long ldx, long gsx,
+                                     long ldy, long gsy, int epilogue, int f32, void* stream) {
+  if (ldx <= 0 || ldy <= 0 || gsx < 0 || gsy < 0) return SSD_ERR_SHAPE;
+  return launch(x_rows, w_rows, y, M, N, K, epilogue, nullptr, 0, nullptr, 1, f32, stream, G, ldx, gsx, ldy, gsy);
 }

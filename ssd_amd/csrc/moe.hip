@@ -1,6 +1,9 @@
 // Routed feed-forward (mixture of experts) around the grouped GEMM of gemm_rows.hip:
 //   ssd_moe_route    from the router's fp32 logits z = W_r h (a GEMM with fp32 rows out): the `top` largest per token (lowest index
 //                    wins a tie) and the softmax over them
+//   ssd_moe_route_softmax  the other common router: scores = softmax over ALL experts, experts in contiguous groups of which only the
+//                    best `keep` (by their largest score) stay eligible, the `top` largest eligible scores, divided by their sum
+//                    (+ 1e-20) and multiplied by a constant
 //   ssd_moe_plan     counting sort of the T * top (token, slot) pairs by expert: offsets[E+1], perm (sorted row -> pair), inv (pair -> sorted row)
 //   ssd_moe_combine  out[t] = sum_j weight[t][j] * y[inv[t * top + j]] (+ shared[t]) in slot order, fp32
 // Between plan and combine the caller runs the experts as two grouped GEMMs over the sorted rows (up with the activation as epilogue,
@@ -36,6 +39,62 @@ moe_route_kernel(const float* __restrict__ zin, int32_t* __restrict__ idx, float
     __syncthreads();
   }
   if (lane < top) wt[(size_t)t * top + lane] = myval / den;
+}
+
+// Softmax-then-top-k routing with group-limited choice.  One wave per token; logits row stride ldz (other per-token logits may share the
+// row).  Among equal scores the lowest index wins, for groups and for experts.
+__global__ void __launch_bounds__(64)
+moe_route_softmax_kernel(const float* __restrict__ zin, long ldz, int32_t* __restrict__ idx, float* __restrict__ wt, int E, int top,
+                         int groups, int keep, float scale) {
+  extern __shared__ float z[];      // [E] scores, then [groups] group scores
+  float* gs = z + E;
+  const int t = blockIdx.x, lane = threadIdx.x;
+  float mx = -INFINITY;
+  for (int e = lane; e < E; e += 64) { const float v = zin[(size_t)t * ldz + e]; z[e] = v; mx = fmaxf(mx, v); }
+  mx = wave_max(mx);
+  float den = 0.f;
+  for (int e = lane; e < E; e += 64) { const float p = expf(z[e] - mx); z[e] = p; den += p; }
+  den = wave_sum(den);
+  for (int e = lane; e < E; e += 64) z[e] = z[e] / den;
+  __syncthreads();
+  if (groups > 1 && keep < groups) {
+    const int per = E / groups;
+    for (int g = lane; g < groups; g += 64) {
+      float b = -INFINITY;
+      for (int i = 0; i < per; ++i) b = fmaxf(b, z[g * per + i]);
+      gs[g] = b;
+    }
+    __syncthreads();
+    // `keep` rounds of a wave-wide argmax over the groups; a kept group is marked by a score of +inf
+    for (int j = 0; j < keep; ++j) {
+      float best = -INFINITY; int bi = 0x7fffffff;
+      for (int g = lane; g < groups; g += 64) { const float v = gs[g]; if (v != INFINITY && v > best) { best = v; bi = g; } }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, 64); const int oi = __shfl_xor(bi, o, 64);
+        if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+      }
+      if (lane == 0 && bi != 0x7fffffff) gs[bi] = INFINITY;
+      __syncthreads();
+    }
+    for (int e = lane; e < E; e += 64) if (gs[e / per] != INFINITY) z[e] = -1.0f;       // not eligible (scores are >= 0)
+    __syncthreads();
+  }
+  float sum = 0.f, myval = 0.f;
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY; int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) { const float v = z[e]; if (v > best) { best = v; bi = e; } }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(best, o, 64); const int oi = __shfl_xor(bi, o, 64);
+      if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+    }
+    sum += best;
+    if (lane == j % 64) { myval = best; idx[(size_t)t * top + j] = bi; }
+    if (lane == 0) z[bi] = -2.0f;
+    __syncthreads();
+  }
+  if (lane < top) wt[(size_t)t * top + lane] = myval / (sum + 1e-20f) * scale;
 }
 
 __global__ void __launch_bounds__(1024)
@@ -79,6 +138,17 @@ extern "C" int ssd_moe_route(const float* logits, int32_t* idx, float* weights, 
   if (!logits || !idx || !weights) return SSD_ERR_ARG;
   if (T <= 0 || E <= 0 || E > MOE_MAX_E || top <= 0 || top > E || top > MOE_MAX_TOP) return SSD_ERR_SHAPE;
   hipLaunchKernelGGL(moe_route_kernel, dim3(T), dim3(64), E * sizeof(float), (hipStream_t)stream, logits, idx, weights, E, top);
+  return LAUNCH_OK();
+}
+
+extern "C" int ssd_moe_route_softmax(const float* logits, long ld, int32_t* idx, float* weights, int T, int E, int top, int groups,
+                                     int keep, float scale, void* stream) {
+  if (!logits || !idx || !weights) return SSD_ERR_ARG;
+  if (T <= 0 || E <= 0 || E > MOE_MAX_E || top <= 0 || top > MOE_MAX_TOP || ld < E || groups <= 0 || E % groups || keep <= 0 ||
+      keep > groups || top > (E / groups) * keep)
+    return SSD_ERR_SHAPE;
+  hipLaunchKernelGGL(moe_route_softmax_kernel, dim3(T), dim3(64), (E + groups) * sizeof(float), (hipStream_t)stream, logits, ld, idx,
+                     weights, E, top, groups, keep, scale);
   return LAUNCH_OK();
 }
 

@@ -31,10 +31,15 @@ class Block:
 
 class BlockManager:
     def __init__(self, num_blocks: int, block_size: int, is_draft: bool = False, speculate_k: int = -1,
-                 max_model_len: int = -1, verbose: bool = False, prefix_cache: bool = True):
+                 max_model_len: int = -1, verbose: bool = False, prefix_cache: bool = True, state_slots: int = 0):
         """prefix_cache=False: every allocation takes fresh blocks (EAGLE-3: the draft's KV row p belongs to token p+1 and
-        is conditioned on the target activation of position p, which a prefix hit would neither compute nor align)."""
+        is conditioned on the target activation of position p, which a prefix hit would neither compute nor align).
+        state_slots > 0: the model also keeps a recurrent state per live sequence; a sequence takes one of that many slots with its
+        blocks and returns it with them (lowest free slot first).  A state is not a function of cached pages, so such models run
+        with prefix_cache=False."""
         assert num_blocks > 0
+        assert not (state_slots and prefix_cache), "recurrent state cannot be rebuilt from cached pages"
+        self.free_state_slots: list[int] | None = list(range(state_slots)) if state_slots else None
         self.prefix_cache = prefix_cache
         self.block_size = block_size
         self.is_draft = is_draft
@@ -80,11 +85,16 @@ class BlockManager:
 
     # ---- whole-sequence allocation with prefix reuse (reference :99-127) ----
     def can_allocate(self, seq) -> bool:
+        if self.free_state_slots is not None and not self.free_state_slots:
+            return False
         return len(self.free_block_ids) >= seq.num_blocks
 
     def allocate(self, seq) -> None:
         table = self._table(seq)
         assert not table
+        if self.free_state_slots is not None:
+            assert seq.state_slot < 0
+            seq.state_slot = self.free_state_slots.pop(0)
         h, missed = -1, not self.prefix_cache
         for i in range(seq.num_blocks):
             toks = seq.block(i)
@@ -123,6 +133,10 @@ class BlockManager:
         else:
             seq.num_cached_tokens = 0
         table.clear()
+        if self.free_state_slots is not None and seq.state_slot >= 0:
+            import bisect
+            bisect.insort(self.free_state_slots, seq.state_slot)
+            seq.state_slot = -1
 
     # ---- lookahead reservation for decode / speculation (reference :137-176) ----
     def _blocks_for(self, seq, lookahead: int) -> int:

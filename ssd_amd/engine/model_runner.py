@@ -34,6 +34,9 @@ def model_class(family: str):
     if family == "fatulix":
         from ssd_amd.fatulix import HipFatulix
         return HipFatulix
+    if family == "zerusun":
+        from ssd_amd.zerusun import HipZerusun
+        return HipZerusun
     return HipDecoder
 
 
@@ -121,6 +124,8 @@ class ModelRunner:
         self.d_cu_q = torch.zeros(B + 1, dtype=torch.int32, **dev)
         self.d_gather = torch.zeros(B, dtype=torch.int32, **dev)
         self.d_bt = torch.zeros(B, self.max_blocks, dtype=torch.int32, **dev)
+        # recurrent-state slots of the batch's sequences (models with recurrent layers; the block manager hands the slots out)
+        self.d_state = torch.zeros(B, dtype=torch.int32, **dev) if getattr(self.model, "state_slots", 0) else None
         self.d_next = torch.zeros(max(self.max_decode_tokens, B), dtype=torch.int64, **dev)
         self.d_spec = torch.zeros(B, self.K + 1, dtype=torch.int64, **dev)
         self.d_step = torch.zeros(1, dtype=torch.int32, **dev)
@@ -266,6 +271,10 @@ class ModelRunner:
             dst[:n].copy_(stage[:n], non_blocking=True)
 
     def _upload_block_tables(self, seqs) -> None:
+        if self.d_state is not None:
+            slots = [s.state_slot for s in seqs]
+            assert all(0 <= x < self.model.state_slots for x in slots), "a sequence of a recurrent model runs without a state slot"
+            self._upload(self.d_state, slots, torch.int32)
         rows = []
         for s in seqs:
             t = self._table(s)
@@ -351,9 +360,11 @@ class ModelRunner:
     def _meta(self, kind: str, B: int, max_q: int = 1, tree_step: int = 0) -> AttnMeta:
         hint = self._ctx_hint
         if kind == "prefill":
-            return AttnMeta(H.MODE_CAUSAL, B, max_q, self.d_slots, self.d_ctx, self.d_bt, cu_q=self.d_cu_q, ctx_hint=hint)
+            return AttnMeta(H.MODE_CAUSAL, B, max_q, self.d_slots, self.d_ctx, self.d_bt, cu_q=self.d_cu_q, ctx_hint=hint,
+                            state_slots=self.d_state)
         if kind == "decode":
-            return AttnMeta(H.MODE_CAUSAL, B, 1, self.d_slots, self.d_ctx, self.d_bt, q_per_seq=1, ctx_hint=hint)
+            return AttnMeta(H.MODE_CAUSAL, B, 1, self.d_slots, self.d_ctx, self.d_bt, q_per_seq=1, ctx_hint=hint,
+                            state_slots=self.d_state)
         if kind == "verify":
             return AttnMeta(H.MODE_CAUSAL, B, self.K + 1, self.d_slots, self.d_ctx, self.d_bt, q_per_seq=self.K + 1, ctx_hint=hint)
         raise ValueError(kind)

@@ -33,8 +33,11 @@ class Scheduler:
         self.block_size = config.kvcache_block_size
         self.MQ_LEN = sum(config.fan_out_list) if (config.speculate and config.draft_async) else 0
         pc = not getattr(config, "use_eagle", False)
+        # a model with recurrent layers: one state slot per live sequence (max_num_seqs of them), no prefix reuse
+        recurrent = bool(getattr(config.hf_config, "recurrent", False))
         self.block_manager = BlockManager(config.num_kvcache_blocks, self.block_size, is_draft=False,
-                                          max_model_len=self.max_model_len, prefix_cache=pc)
+                                          max_model_len=self.max_model_len, prefix_cache=pc and not recurrent,
+                                          state_slots=self.max_num_seqs if recurrent else 0)
         self.draft_block_manager = None
         if self.speculate:
             assert draft_num_blocks is not None and draft_num_blocks > 0

@@ -33,6 +33,7 @@ class Sequence:
         self.num_draft_cached_tokens = 0
         self.block_table: list[int] = []
         self.draft_block_table: list[int] = []
+        self.state_slot = -1            # recurrent-state slot (models with recurrent layers), held from admission to release
         self.last_spec_step_accepted_len = -1
         self.recovery_token_id: int | None = None
         # the prefill's token once LLMEngine.generate handed it to the stream ahead of the first speculation round; consumed

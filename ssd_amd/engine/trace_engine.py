@@ -2,7 +2,8 @@
 portions of any size beside single tokens of other requests, all entries of a step as ONE varlen batch -- and the fp32 logits of the
 asked positions come back; nothing is sampled.  The schedule is the caller's (a trace names what runs in which step), everything
 else is the generation path's: Config, ModelRunner (weights, paged KV cache, staging, forward, LM head), BlockManager (pages are
-taken at admission and as a request grows, and given back when it ends, so pages are used again) and Sequence.
+taken at admission and as a request grows, and given back when it ends, so pages are used again; a model with recurrent layers
+also gets one of `max_live` state slots per request from it) and Sequence.
 
 Prefix caching is off here: a trace asks for logits at given positions, and a position served from another request's pages is
 never computed."""
@@ -34,7 +35,9 @@ class TraceEngine:
                                       num_kvcache_blocks=pool)
         else:
             self.runner = runner_factory(self.config)
-        self.blocks = BlockManager(pool, block_size, max_model_len=cap, prefix_cache=False)
+        # a model with recurrent layers: max_live state slots, taken and returned with a request's pages
+        recurrent = bool(getattr(self.config.hf_config, "recurrent", False))
+        self.blocks = BlockManager(pool, block_size, max_model_len=cap, prefix_cache=False, state_slots=max_live if recurrent else 0)
         self.live: dict[str, Sequence] = {}
 
     def step(self, entries: list[dict], end: list[str] = ()) -> torch.Tensor | None:

@@ -20,12 +20,12 @@ import torch
 from ssd_amd.hip import ops as H
 from ssd_amd.model import AttnMeta
 from ssd_amd.model_config import FatulixConfig
+from ssd_amd.res32 import Res32Decoder
 
 BF16 = torch.bfloat16
 
 
-class HipFatulix:
-    supports_float32 = True
+class HipFatulix(Res32Decoder):
 
     def __init__(self, cfg: FatulixConfig, *, max_tokens: int, max_seqs: int, max_blocks: int, block_size: int, max_model_len: int,
                  device: torch.device, tp_rank: int = 0, tp_size: int = 1, tp_group=None, max_logit_rows: int | None = None,
@@ -110,14 +110,6 @@ class HipFatulix:
                 if lc.mlp.shared_ff:
                     w[p + "mlp.shared.up"] = cv(raw[p + "mlp.shared.up"])
                     w[p + "mlp.shared.down"] = cv(raw[p + "mlp.shared.down"])
-        torch.cuda.synchronize(self.device)
-
-    def overwrite_weights(self, weight_iter) -> None:
-        old, self.w = self.w, {}
-        self.load_weights(weight_iter)
-        new, self.w = self.w, old
-        for n, t in new.items():
-            old[n].copy_(t)
         torch.cuda.synchronize(self.device)
 
     def weight_bytes(self) -> int:
@@ -239,16 +231,3 @@ class HipFatulix:
         H.gemm_rows(self.lastn, self.w["head"], self.logits32, n, self.V, self.W, self.f32)
         H.rows_f32_to_bf16(self.logits32, self.logits, n, self.V, self.V, self.Vp)
         return n
-
-    def has_argmax_parts(self, n: int) -> bool:
-        return False
-
-    def argmax(self, n: int, out: torch.Tensor, out2: torch.Tensor | None = None, out3=None, out3_stride: int = 0) -> None:
-        assert out3 is None
-        H.argmax_rows(self.logits, self.Vp, n, self.V, out, out2)
-
-    def full_logits(self, n: int) -> torch.Tensor:
-        return self.logits[:n] if self.Vp == self.V else self.logits[:n, :self.V].contiguous()
-
-    def logits_f32(self, n: int) -> torch.Tensor:
-        return self.logits32[:n]

@@ -16,7 +16,7 @@ _LIB = None
 
 c_void_p, c_int, c_long, c_float, c_int64 = C.c_void_p, C.c_int, C.c_long, C.c_float, C.c_int64
 
-ABI_VERSION = 3       # include/ssd_hip.h SSD_HIP_ABI_VERSION (tests/test_abi.py compares the two)
+ABI_VERSION = 4       # include/ssd_hip.h SSD_HIP_ABI_VERSION (tests/test_abi.py compares the two)
 
 # name -> argtypes, exactly include/ssd_hip.h (+ include/ssd_hip_tune.h)
 SIGNATURES = {
@@ -126,6 +126,21 @@ SIGNATURES = {
     "ssd_moe_route": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ssd_moe_plan": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
     "ssd_moe_combine": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ssd_gemm_rows_batched": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_long, c_int, c_int, c_void_p],
+    "ssd_dyt_embed": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_long, c_int,
+                      c_void_p],
+    "ssd_dyt_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ssd_parallel_tail": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_long, c_void_p, c_void_p,
+                          c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_void_p],
+    "ssd_glu_rows": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "ssd_latent_store": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_float, c_int,
+                         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "ssd_latent_attn": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                        c_int, c_int, c_int, c_int, c_float, c_void_p, c_float, c_int, c_void_p, c_int, c_void_p],
+    "ssd_lightning_scan": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                           c_int, c_int, c_int, c_int, c_void_p],
+    "ssd_lightning_gate_norm": [c_void_p, c_void_p, c_long, c_int, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ssd_moe_route_softmax": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "ssd_draft_advance": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int,
                           c_void_p, c_int, c_void_p],
 }

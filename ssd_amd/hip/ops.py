@@ -447,3 +447,68 @@ def moe_plan(idx, T: int, top: int, E: int, offsets, perm, inv):
 
 def moe_combine(y, inv, weights, shared, out, T: int, top: int, W: int):
     _check(load_library().ssd_moe_combine(_p(y), _p(inv), _p(weights), _p(shared), _p(out), T, top, W, _stream()), "ssd_moe_combine")
+
+
+def gemm_rows_batched(x, w, y, M: int, N: int, K: int, G: int, ldx: int, gsx: int, ldy: int, gsy: int, f32: bool, epilogue: int = GR_F32):
+    """G products in one launch: group g reads x + g * gsx (row stride ldx), w[g] ([N][K]) and writes y + g * gsy (row stride ldy)."""
+    _check(load_library().ssd_gemm_rows_batched(_p(x), _p(w), _p(y), M, N, K, G, ldx, gsx, ldy, gsy, epilogue, int(f32), _stream()),
+           "ssd_gemm_rows_batched")
+
+
+# ---- parallel layers with Dynamic-Tanh norms, latent attention, linear attention over a recurrent state ----
+
+GLU_SILU, GLU_GELU_TANH = 0, 1
+
+
+def dyt_embed(ids, table, alpha, weight, bias, x, x0, cat, ld_cat: int, T: int, W: int, f32: bool):
+    _check(load_library().ssd_dyt_embed(_p(ids), _p(table), _p(alpha), _p(weight), _p(bias), _p(x), _p(x0), _p(cat), ld_cat, T, W,
+                                        table.shape[0], int(f32), _stream()), "ssd_dyt_embed")
+
+
+def dyt_rows(x, alpha, weight, bias, out_rows, T: int, W: int, f32: bool, add_vec=None, gather=None):
+    _check(load_library().ssd_dyt_rows(_p(x), _p(add_vec), _p(alpha), _p(weight), _p(bias), _p(out_rows), _p(gather), T, W, int(f32),
+                                       _stream()), "ssd_dyt_rows")
+
+
+def parallel_tail(x, y_mix, T: int, W: int, f32: bool, *, y_ff=None, ydn=None, inv=None, weights=None, top: int = 0, shared=None,
+                  shared_gate=None, ld_shared_gate: int = 0, next_alpha=None, next_weight=None, next_bias=None, next_out=None, cat=None,
+                  ld_cat: int = 0):
+    """x += y_mix + (y_ff | routed mix of ydn + sigmoid(shared_gate) * shared | 0); next_out = dyt(x); cat = x as element-type rows."""
+    _check(load_library().ssd_parallel_tail(_p(x), _p(y_mix), _p(y_ff), _p(ydn), _p(inv), _p(weights), top, _p(shared), _p(shared_gate),
+                                            ld_shared_gate, _p(next_alpha), _p(next_weight), _p(next_bias), _p(next_out), _p(cat), ld_cat,
+                                            T, W, int(f32), _stream()), "ssd_parallel_tail")
+
+
+def glu_rows(ab, out_rows, rows: int, F: int, act: int, f32: bool):
+    _check(load_library().ssd_glu_rows(_p(ab), _p(out_rows), rows, F, act, int(f32), _stream()), "ssd_glu_rows")
+
+
+def latent_store(proj, ld: int, q_rank: int, kv_rank: int, rot: int, H: int, q_norm_w, kv_norm_w, eps: float, positions, freqs,
+                 mag: float, rot_dims: int, slots, cq_out, cache, gate_out, T: int, f32: bool):
+    _check(load_library().ssd_latent_store(_p(proj), ld, q_rank, kv_rank, rot, H, _p(q_norm_w), _p(kv_norm_w), eps, _p(positions),
+                                           _p(freqs), mag, rot_dims, _p(slots), _p(cq_out), _p(cache), _p(gate_out), T, int(f32),
+                                           _stream()), "ssd_latent_store")
+
+
+def latent_attn(q_abs, q_rows, cache, gate, block_tables, max_blocks: int, positions, B: int, T: int, H: int, D: int, rot: int,
+                kv_rank: int, block_size: int, window: int, scale: float, freqs, mag: float, rot_dims: int, out_rows, f32: bool,
+                cu_q=None, q_per_seq: int = 0):
+    _check(load_library().ssd_latent_attn(_p(q_abs), _p(q_rows), _p(cache), _p(gate), _p(block_tables), max_blocks, _p(positions),
+                                          _p(cu_q), q_per_seq, B, T, H, D, rot, kv_rank, block_size, window, scale, _p(freqs), mag,
+                                          rot_dims, _p(out_rows), int(f32), _stream()), "ssd_latent_attn")
+
+
+def lightning_scan(proj, ld: int, q_off: int, k_off: int, v_off: int, decay, positions, state_slots, state, out_rows, B: int, H: int,
+                   D: int, Dv: int, cu_q=None, q_per_seq: int = 0):
+    _check(load_library().ssd_lightning_scan(_p(proj), ld, q_off, k_off, v_off, _p(decay), _p(positions), _p(cu_q), q_per_seq,
+                                             _p(state_slots), _p(state), _p(out_rows), B, H, D, Dv, _stream()), "ssd_lightning_scan")
+
+
+def lightning_gate_norm(o_rows, proj, ld: int, g_off: int, weight, eps: float, out_rows, T: int, N: int, f32: bool):
+    _check(load_library().ssd_lightning_gate_norm(_p(o_rows), _p(proj), ld, g_off, _p(weight), eps, _p(out_rows), T, N, int(f32),
+                                                  _stream()), "ssd_lightning_gate_norm")
+
+
+def moe_route_softmax(logits, ld: int, idx, weights, T: int, E: int, top: int, groups: int, keep: int, scale: float):
+    _check(load_library().ssd_moe_route_softmax(_p(logits), ld, _p(idx), _p(weights), T, E, top, groups, keep, scale, _stream()),
+           "ssd_moe_route_softmax")

@@ -42,6 +42,7 @@ class AttnMeta:
     tree_F: int = 1
     tree_jidx: torch.Tensor | None = None
     ctx_hint: int = 0             # host-side upper bound of the context lengths (0 = unknown -> max_model_len)
+    state_slots: torch.Tensor | None = None     # int32 [B]: recurrent-state slot of every sequence (models with recurrent layers)
 
 
 def make_cos_sin(head_dim: int, max_pos: int, theta: float, device) -> torch.Tensor:

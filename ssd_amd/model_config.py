@@ -185,8 +185,174 @@ class FatulixConfig:
         return out
 
 
+# --------------------------------------------------------------------------------------------------
+# Zerusun: parallel layers with Dynamic-Tanh norms; mixers are latent attention (sliding window) or linear attention with decay
+# --------------------------------------------------------------------------------------------------
+@dataclass
+class RopeSpec:
+    """Rotary positions on the first `dims` entries of a rotated part ("rotate half" pairing: i with i + dims / 2), frequencies
+    base^(-2i/dims); scaling (optional) = YaRN: {factor, original, fast, slow}."""
+    dims: int
+    base: float
+    scaling: dict | None = None
+
+    def frequencies(self) -> tuple[list[float], float]:
+        """(per-pair angular frequencies, the factor cos and sin carry).  YaRN keeps the pairs that turn more than `fast` times over
+        `original` positions, divides the frequency of those that turn fewer than `slow` times by `factor`, and blends linearly
+        between the two corner pairs; cos and sin are scaled by 0.1 ln(factor) + 1."""
+        import math
+        half = self.dims // 2
+        f = [self.base ** (-2.0 * i / self.dims) for i in range(half)]
+        sc = self.scaling
+        if not sc:
+            return f, 1.0
+        factor, orig = float(sc["factor"]), float(sc["original"])
+        corner = lambda turns: self.dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(self.base))
+        lo = max(math.floor(corner(float(sc["fast"]))), 0)
+        hi = min(math.ceil(corner(float(sc["slow"]))), self.dims - 1)
+        ramp = [min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0) for i in range(half)]
+        return [fi / factor * r + fi * (1.0 - r) for fi, r in zip(f, ramp)], 0.1 * math.log(factor) + 1.0
+
+
+@dataclass
+class LatentAttention:
+    """Attention whose queries and keys / values pass through low-rank latents; per head `dim` unrotated + `rot_dim` rotated query / key
+    entries (the rotated key part is shared by all heads), value size `vdim`; only the kv latent and the rotated key part are cached.
+    window: a token sees itself and the window - 1 tokens before it (0: every earlier token).  Per-head sigmoid output gate."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    window: int
+    rope: RopeSpec
+    kind: str = "latent_attention"
+
+
+@dataclass
+class LightningAttention:
+    """Linear attention with a per-head scalar decay over a recurrent [dim][vdim] state; silu on q, k, v; RMS norm over the concatenated
+    heads and an elementwise sigmoid gate before the output projection."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: list = field(default_factory=list)
+    kind: str = "lightning"
+
+
+@dataclass
+class GluMLP:
+    """Dense gated feed-forward W_down(act(W_gate h) * W_up h), act = tanh-form gelu."""
+    ff: int
+    kind: str = "dense"
+
+
+@dataclass
+class GroupRoutedMLP:
+    """Mixture of gated (silu) experts: softmax over all experts, `groups` contiguous groups of which the best `keep` stay eligible,
+    the `top` largest scores renormalised and multiplied by `scale`; optional shared expert with a per-token sigmoid gate."""
+    experts: int
+    top: int
+    ff: int
+    groups: int = 1
+    keep: int = 1
+    scale: float = 1.0
+    shared_ff: int = 0
+    kind: str = "moe"
+
+
+@dataclass
+class ZerusunLayer:
+    mixer: object               # LatentAttention | LightningAttention
+    mlp: object                 # GluMLP | GroupRoutedMLP | None
+
+
+@dataclass
+class ZerusunConfig:
+    """config.json keys: architecture, vocab, width, norm.eps, layers[{type, mixer{...}, mlp{kind, ...} | null}], loop{start, stop, times}.
+    Layers [start, stop) run `times` passes with the same weights (each pass with cache pages / state of its own); before the first layer
+    of EVERY pass x <- W_in [x; x0] + step[pass], x0 = the embedding output."""
+    vocab_size: int
+    hidden_size: int
+    rms_norm_eps: float
+    layers: list = field(default_factory=list)
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1
+    family: str = "zerusun"
+    max_position_embeddings: int = 1 << 20
+    tie_word_embeddings: bool = True
+
+    def runs(self) -> list[tuple[int, int]]:
+        """(layer, pass) of every layer run in execution order."""
+        a, b = self.loop_start, self.loop_stop
+        if b <= a:
+            return [(i, 0) for i in range(len(self.layers))]
+        span = [(i, ps) for ps in range(self.loop_times) for i in range(a, b)]
+        return [(i, 0) for i in range(a)] + span + [(i, 0) for i in range(b, len(self.layers))]
+
+    @property
+    def has_loop(self) -> bool:
+        return self.loop_stop > self.loop_start
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.runs())
+
+    @property
+    def recurrent(self) -> bool:
+        """True when some layer keeps a per-sequence state that is not a function of cached pages: no prefix caching, and every live
+        sequence holds a state slot."""
+        return any(l.mixer.kind == "lightning" for l in self.layers)
+
+    def to_dict(self) -> dict:
+        return asdict(self)
+
+    @staticmethod
+    def from_json(cfg: dict) -> "ZerusunConfig":
+        layers = []
+        for lc in cfg["layers"]:
+            m, kind = lc["mixer"], lc["type"]
+            if kind == "latent_attention":
+                r = m["rot"]
+                rope = RopeSpec(int(r["dims"]), float(r["base"]), dict(r["scaling"]) if r.get("scaling") else None)
+                mask = m.get("mask") or {}
+                mixer = LatentAttention(int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]), int(m["q_rank"]),
+                                        int(m["kv_rank"]), float(m["scale"]), int(mask.get("size") or 0), rope)
+                if rope.dims % 2 or rope.dims > mixer.rot_dim:
+                    raise ValueError("Zerusun: rot.dims must be even and at most rot_dim")
+            elif kind == "lightning":
+                mixer = LightningAttention(int(m["heads"]), int(m["dim"]), int(m["vdim"]), [float(d) for d in m["decay"]])
+                if len(mixer.decay) != mixer.heads:
+                    raise ValueError("Zerusun: one decay per head")
+            else:
+                raise ValueError(f"Zerusun: unknown layer type {kind!r}")
+            ml = lc.get("mlp")
+            mlp = None
+            if ml is not None:
+                if ml["kind"] == "dense":
+                    mlp = GluMLP(int(ml["ff"]))
+                elif ml["kind"] == "moe":
+                    r, g, sh = ml["router"], ml["router"].get("groups") or {}, ml.get("shared")
+                    mlp = GroupRoutedMLP(int(r["experts"]), int(r["top"]), int(ml["expert"]["ff"]), int(g.get("count", 1)),
+                                         int(g.get("keep", 1)), float(r.get("scale", 1.0)), int(sh["ff"]) if sh else 0)
+                    if mlp.experts % mlp.groups or not (1 <= mlp.keep <= mlp.groups) or mlp.top > mlp.experts // mlp.groups * mlp.keep:
+                        raise ValueError("Zerusun: router groups do not fit the experts")
+                else:
+                    raise ValueError(f"Zerusun: unknown feed-forward kind {ml['kind']!r}")
+            layers.append(ZerusunLayer(mixer, mlp))
+        loop = cfg.get("loop") or {}
+        out = ZerusunConfig(int(cfg["vocab"]), int(cfg["width"]), float(cfg["norm"]["eps"]), layers, int(loop.get("start", 0)),
+                            int(loop.get("stop", 0)), int(loop.get("times", 1)))
+        if not (0 <= out.loop_start and out.loop_stop <= len(layers)) or out.loop_times < 1:
+            raise ValueError("Zerusun: loop out of range")
+        return out
+
+
 # config.json "architecture" values that are read by this package's own readers (everything else goes through transformers' AutoConfig)
-ARCHITECTURES = {"Fatulix": FatulixConfig.from_json}
+ARCHITECTURES = {"Fatulix": FatulixConfig.from_json, "Zerusun": ZerusunConfig.from_json}
 
 
 def read_native_config(model_dir: str):

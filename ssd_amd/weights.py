@@ -69,11 +69,47 @@ def fatulix_param_shapes(cfg) -> list[tuple[str, tuple[int, ...]]]:
     return out
 
 
+def zerusun_param_shapes(cfg) -> list[tuple[str, tuple[int, ...]]]:
+    """Tensor names and shapes of a Zerusun checkpoint (model_config.ZerusunConfig).  A Dynamic-Tanh norm 'n' is three tensors: 'n'
+    (weight), 'n.b' (bias), 'n.alpha' (a scalar)."""
+    W = cfg.hidden_size
+    norm = lambda n: [(n, (W,)), (n + ".b", (W,)), (n + ".alpha", ())]
+    glu = lambda p, ff: [(p + "gate", (ff, W)), (p + "up", (ff, W)), (p + "down", (W, ff))]
+    out = [("embed", (cfg.vocab_size, W))] + norm("embed.norm")
+    if cfg.has_loop:
+        out += [("loop.in", (W, 2 * W)), ("loop.step", (cfg.loop_times, W))]
+    for i, lc in enumerate(cfg.layers):
+        p, m = f"l{i}.", lc.mixer
+        out += norm(p + "norm1")
+        if m.kind == "latent_attention":
+            out += [(p + "mix.dq", (m.q_rank, W)), (p + "mix.dq.norm", (m.q_rank,)), (p + "mix.uq", (m.heads * (m.dim + m.rot_dim), m.q_rank)),
+                    (p + "mix.dkv", (m.kv_rank + m.rot_dim, W)), (p + "mix.dkv.norm", (m.kv_rank,)),
+                    (p + "mix.uk", (m.heads * m.dim, m.kv_rank)), (p + "mix.uv", (m.heads * m.vdim, m.kv_rank)),
+                    (p + "mix.g", (m.heads, W)), (p + "mix.o", (W, m.heads * m.vdim))]
+        else:
+            out += [(p + "mix.q", (m.heads * m.dim, W)), (p + "mix.k", (m.heads * m.dim, W)), (p + "mix.v", (m.heads * m.vdim, W)),
+                    (p + "mix.g", (m.heads * m.vdim, W)), (p + "mix.o", (W, m.heads * m.vdim)), (p + "mix.norm", (m.heads * m.vdim,))]
+        ml = lc.mlp
+        if ml is None:
+            continue
+        if ml.kind == "dense":
+            out += glu(p + "mlp.", ml.ff)
+        else:
+            for e in range(ml.experts):
+                out += glu(p + f"mlp.e{e}.", ml.ff)
+            out.append((p + "mlp.router", (ml.experts, W)))
+            if ml.shared_ff:
+                out += glu(p + "mlp.shared.", ml.shared_ff) + [(p + "mlp.shared.sg", (1, W))]
+    return out + norm("final.norm")
+
+
 def param_shapes(cfg: ModelConfig) -> list[tuple[str, tuple[int, ...]]]:
     if cfg.family == "eagle3":
         return eagle_param_shapes(cfg)
     if cfg.family == "fatulix":
         return fatulix_param_shapes(cfg)
+    if cfg.family == "zerusun":
+        return zerusun_param_shapes(cfg)
     h, hd, nh, nkv, I, V = cfg.hidden_size, cfg.head_dim, cfg.num_heads, cfg.num_kv_heads, cfg.intermediate_size, cfg.vocab_size
     out = [("model.embed_tokens.weight", (V, h))]
     for i in range(cfg.num_layers):
@@ -286,6 +322,10 @@ def synthetic_tensor(name: str, shape, seed: int, std: float, gen_device: str, n
         gc.manual_seed(_name_seed(seed, name))
         idx = torch.randperm(V, generator=gc)[:shape[0]].sort().values
         return (idx - torch.arange(shape[0])).to(torch.int64).to(gen_device)
+    if name.endswith(".alpha"):     # Dynamic-Tanh norms: the scalar inside the tanh; its bias is the '.b' tensor
+        return torch.full(shape, 0.5, dtype=BF16, device=gen_device)
+    if name.endswith(".b"):
+        return torch.zeros(shape, dtype=BF16, device=gen_device)
     if "norm" in name or name.endswith("_ln.weight"):
         if norm_jitter == 0.0:
             return torch.ones(shape, dtype=BF16, device=gen_device)

@@ -34,7 +34,7 @@ class Scheduler:
         self.MQ_LEN = sum(config.fan_out_list) if (config.speculate and config.draft_async) else 0
         pc = not getattr(config, "use_eagle", False)
         # a model with recurrent layers: one state slot per live sequence (max_num_seqs of them), no prefix reuse
-        recurrent = bool(getattr(config.hf_config, "recurrent", False))
+        recurrent = bool(getattr(getattr(config, "hf_config", None), "recurrent", False))
         self.block_manager = BlockManager(config.num_kvcache_blocks, self.block_size, is_draft=False,
                                           max_model_len=self.max_model_len, prefix_cache=pc and not recurrent,
                                           state_slots=self.max_num_seqs if recurrent else 0)

@@ -164,3 +164,97 @@ def forward(cfg: dict, weights: dict, tokens, taps: list | None = None):
         if taps is not None:
             taps.append(x.clone())
     return norm(x, "final.norm") @ P["embed"].T
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# small self-made models for the tests
+# ---------------------------------------------------------------------------------------------------------------------
+def latent_layer(heads=4, dim=16, rot_dim=8, vdim=24, q_rank=40, kv_rank=48, window=9, scale=None, rot_dims=None, base=10000.0,
+                 scaling="yarn", mlp=None) -> dict:
+    sc = {"factor": 4.0, "original": 64, "fast": 32.0, "slow": 1.0} if scaling == "yarn" else scaling
+    return {"type": "latent_attention", "mlp": mlp,
+            "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "q_rank": q_rank, "kv_rank": kv_rank,
+                      "scale": scale if scale is not None else (dim + rot_dim) ** -0.5, "mask": {"size": window} if window else None,
+                      "rot": {"dims": rot_dims or rot_dim, "base": base, "scaling": sc}}}
+
+
+def lightning_layer(heads=3, dim=16, vdim=24, decay=None, mlp=None) -> dict:
+    decay = decay or [math.exp(-1.0 / (2.0 ** (1 + 1.5 * h))) for h in range(heads)]
+    return {"type": "lightning", "mlp": mlp, "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "decay": decay}}
+
+
+def dense_mlp(ff=40) -> dict:
+    return {"kind": "dense", "ff": ff}
+
+
+def moe_mlp(experts=8, top=2, ff=24, groups=(2, 1), scale=1.5, shared_ff=40) -> dict:
+    return {"kind": "moe", "expert": {"ff": ff},
+            "router": {"experts": experts, "top": top, "scale": scale, "groups": {"count": groups[0], "keep": groups[1]} if groups else None},
+            "shared": {"ff": shared_ff} if shared_ff else None}
+
+
+def make_config(layers, vocab=96, width=64, loop=(0, 0, 1), eps=1e-5) -> dict:
+    return {"architecture": "Zerusun", "vocab": vocab, "width": width, "norm": {"eps": eps}, "layers": layers,
+            "loop": {"start": loop[0], "stop": loop[1], "times": loop[2]}}
+
+
+def random_model(cfg: dict, seed: int = 0) -> dict:
+    """bf16 weights of the right shapes for `cfg`: matrices N(0, 1 / fan-in) (queries a little sharper), norm weights around 1."""
+    gen = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+    w = {}
+
+    def mat(name, o, i, gain=1.0):
+        w[name] = (torch.randn(o, i, generator=gen) * gain / math.sqrt(i)).to(torch.bfloat16)
+
+    def vec(name, n, base=1.0, s=0.1):
+        w[name] = (base + s * torch.randn(n, generator=gen)).to(torch.bfloat16)
+
+    def norm(name):
+        vec(name, W)
+        vec(name + ".b", W, 0.0, 0.1)
+        w[name + ".alpha"] = torch.tensor(0.4 + 0.4 * torch.rand((), generator=gen).item()).to(torch.bfloat16)
+
+    def glu_w(p, ff):
+        mat(p + "gate", ff, W, 1.5)
+        mat(p + "up", ff, W, 1.5)
+        mat(p + "down", W, ff)
+
+    mat("embed", cfg["vocab"], W, math.sqrt(W))
+    norm("embed.norm")
+    norm("final.norm")
+    lp = cfg.get("loop") or {}
+    if lp.get("stop", 0) > lp.get("start", 0):
+        mat("loop.in", W, 2 * W, 1.2)
+        w["loop.step"] = (0.3 * torch.randn(lp["times"], W, generator=gen)).to(torch.bfloat16)
+    for i, lc in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", lc["mixer"]
+        norm(p + "norm1")
+        Hh = m["heads"]
+        if lc["type"] == "latent_attention":
+            mat(p + "mix.dq", m["q_rank"], W)
+            vec(p + "mix.dq.norm", m["q_rank"])
+            mat(p + "mix.uq", Hh * (m["dim"] + m["rot_dim"]), m["q_rank"], 3.0)
+            mat(p + "mix.dkv", m["kv_rank"] + m["rot_dim"], W, 1.5)
+            vec(p + "mix.dkv.norm", m["kv_rank"])
+            mat(p + "mix.uk", Hh * m["dim"], m["kv_rank"], 1.5)
+            mat(p + "mix.uv", Hh * m["vdim"], m["kv_rank"])
+            mat(p + "mix.g", Hh, W)
+        else:
+            for n, d in (("q", m["dim"]), ("k", m["dim"]), ("v", m["vdim"]), ("g", m["vdim"])):
+                mat(p + "mix." + n, Hh * d, W, 1.5)
+            vec(p + "mix.norm", Hh * m["vdim"])
+        mat(p + "mix.o", W, Hh * m["vdim"])
+        ml = lc.get("mlp")
+        if ml is None:
+            continue
+        if ml["kind"] == "dense":
+            glu_w(p + "mlp.", ml["ff"])
+            continue
+        for e in range(ml["router"]["experts"]):
+            glu_w(p + f"mlp.e{e}.", ml["expert"]["ff"])
+        mat(p + "mlp.router", ml["router"]["experts"], W, 2.0)
+        if ml.get("shared"):
+            glu_w(p + "mlp.shared.", ml["shared"]["ff"])
+            mat(p + "mlp.shared.sg", 1, W)
+    return w

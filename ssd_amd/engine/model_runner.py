@@ -513,13 +513,17 @@ class ModelRunner:
             return self.model.full_logits(T)
         self._prepare_decode(seqs)
         temps = self._seq_temps(seqs)
+        # the call that captures a graph has already run the step eagerly (the warm-up).  Models whose memory is cache pages run it
+        # once more through the new graph (the same rows land in the same slots); a recurrent state would absorb the token twice,
+        # so such models keep the warm-up's result
+        rerun = not getattr(self.model, "state_slots", 0)
         if any(t > 0 for t in temps):       # autoregressive sampling (AutoRegressiveStep at temperature > 0)
             self._ensure_stochastic()
             self._upload(self.d_temps, temps, torch.float32)
-            if self._launch(("decode_s", B), lambda: self._body_decode(B, False, sample=True)) == "captured":
+            if self._launch(("decode_s", B), lambda: self._body_decode(B, False, sample=True)) == "captured" and rerun:
                 self._prepare_decode(seqs)
                 self.graphs[("decode_s", B, self._ctx_hint)].replay()
-        elif self._launch(("decode", B), lambda: self._body_decode(B, False)) == "captured":
+        elif self._launch(("decode", B), lambda: self._body_decode(B, False)) == "captured" and rerun:
             self._prepare_decode(seqs)
             self.graphs[("decode", B, self._ctx_hint)].replay()
         self._log_margins(B, [(s.seq_id, len(s)) for s in seqs])

@@ -150,12 +150,30 @@ def lib_path() -> str:
     return os.path.join(_PKG, "_lib", "libssdhip.so")
 
 
-def build_library(force: bool = False, quiet: bool = False) -> str:
-    """Compile every HIP source for gfx950 (hipcc cross-compiles without a GPU).  quiet: the build's output goes to stderr."""
+# Translation units that a model family's forward + LM head need (the families that bring their own config.json).  A checkout that
+# has no library yet and serves one of them builds only these, as libssdhip_<family>.so; the full library, once built, takes over.
+_COMMON_ROWS = ["misc.hip", "gemm_rows.hip", "res32.hip", "moe.hip", "sample.hip"]
+FAMILY_SOURCES = {
+    "fatulix": _COMMON_ROWS + ["attention_diff.hip"],
+    "zerusun": _COMMON_ROWS + ["dyt.hip", "attention_latent.hip", "lightning.hip"],
+}
+
+
+def family_lib_path(family: str) -> str:
+    return os.path.join(_PKG, "_lib", f"libssdhip_{family}.so")
+
+
+def build_library(force: bool = False, quiet: bool = False, family: str | None = None) -> str:
+    """Compile every HIP source for gfx950 (hipcc cross-compiles without a GPU).  quiet: the build's output goes to stderr.
+    family: only the translation units of FAMILY_SOURCES[family], linked as libssdhip_<family>.so."""
     src = os.path.join(_PKG, "csrc")
     out = dict(stdout=subprocess.DEVNULL) if quiet else {}
     if force:
         subprocess.check_call(["make", "-C", src, "clean"], **out)
+    if family is not None:
+        subprocess.check_call(["make", "-C", src, "-j8", "SRCS=" + " ".join(FAMILY_SOURCES[family]),
+                               "OUT=../_lib/" + os.path.basename(family_lib_path(family))], **out)
+        return family_lib_path(family)
     subprocess.check_call(["make", "-C", src, "-j8"], **out)
     return lib_path()
 
@@ -164,11 +182,15 @@ class SsdHipError(RuntimeError):
     pass
 
 
-def load_library():
+def load_library(family: str | None = None):
+    """The full library; or, when it has not been built and `family` names one of FAMILY_SOURCES whose library has, that one (the
+    entry points it lacks are simply not bound: calling one raises AttributeError)."""
     global _LIB
     if _LIB is not None:
         return _LIB
-    path = lib_path()
+    path, partial = lib_path(), False
+    if not os.path.exists(path) and family in FAMILY_SOURCES and os.path.exists(family_lib_path(family)):
+        path, partial = family_lib_path(family), True
     if not os.path.exists(path):
         raise SsdHipError(f"{path} not found: build it with `make -C ssd_amd/csrc` (or __graft_entry__.build()); "
                           "there is no CPU fallback for the hot path")
@@ -177,6 +199,8 @@ def load_library():
         try:
             fn = getattr(lib, name)
         except AttributeError as e:
+            if partial:
+                continue
             raise SsdHipError(f"libssdhip.so does not export {name}") from e
         fn.argtypes = args
         fn.restype = c_int
@@ -184,3 +208,11 @@ def load_library():
         raise SsdHipError("libssdhip.so ABI version mismatch")
     _LIB = lib
     return lib
+
+
+def ensure_library(family: str | None = None, quiet: bool = True):
+    """Loads the library, building first what a fresh checkout lacks: the family's translation units for a family of FAMILY_SOURCES,
+    everything otherwise."""
+    if not os.path.exists(lib_path()) and not (family in FAMILY_SOURCES and os.path.exists(family_lib_path(family))):
+        build_library(quiet=quiet, family=family if family in FAMILY_SOURCES else None)
+    return load_library(family)

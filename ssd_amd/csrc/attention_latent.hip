@@ -10,7 +10,7 @@
 // Rotation: the first `rot_dims` of the R rotated entries turn, entry i pairing with i + rot_dims / 2, by angle p * f_i (fp32) with
 // cos and sin scaled by `mag`; f and mag come from the host (they carry the YaRN frequency blend).
 //  * ssd_latent_store  fp32 projection rows [dq | dkv | gate logits] -> c_q rows, the cache row of every token, sigmoid gates
-//  * ssd_latent_attn   scalar fp32 form for any sizes and both element types: a wave owns a (token, head) row, a lane a key for the
+//  * ssd_latent_attn   MFMA form below (bf16, aligned latent sizes), else the scalar fp32 form for any sizes and both element types: a wave owns a (token, head) row, a lane a key for the
 //                      scores and latent columns for the weighted sum; keys in steps of 64 from the window's first key, so a row's
 //                      arithmetic depends on its position alone (not on the portion or the batch it arrives in)
 #include "common.h"
@@ -159,6 +159,175 @@ latent_attn_kernel(const float* __restrict__ q_abs, const T* __restrict__ q_rows
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------------
+// MFMA form (bf16; kv_rank % 32 == 0, rot % 32 == 0, kv_rank <= 512, kv_rank + rot <= 640).  A workgroup owns one token and 16 heads
+// (rows of the score tile = heads: every head reads the SAME cached rows); its NW waves take the 32-key steps of the window round-robin
+// and meet in LDS at the end.  Per step and wave:
+//   S^T[key][head] = K tile x Q      K rows straight from the cache as the A operand (16-byte loads), Q fragments in registers;
+//                                    the two 16-key tiles take the keys in the order (g*8 + r | g*8 + 4 + r), so that a lane ends up
+//                                    with the scores of 8 CONSECUTIVE keys of its head -- already the B operand layout of the next product
+//   online softmax per head          on the accumulator fragments (two cross-lane steps per reduction)
+//   O^T[col][head] += C^T tile x P   the latent part of the K fragments is scattered into LDS transposed ([col][32 keys]) while S is
+//                                    computed, so every cached element is loaded once and the A operand is one 16-byte LDS read
+// Keys outside [first, p] are never loaded (zeros; -inf scores): unwritten cache rows cannot leak.  The steps start at the window's first
+// key, so a row's arithmetic depends on its position alone.
+// ---------------------------------------------------------------------------------------------------------------------
+constexpr int LAT_KT_MAX = 20, LAT_NT_MAX = 32, LAT_CTS = 40;
+
+template <int NW>
+__global__ void __launch_bounds__(NW * 64)
+latent_attn_mfma_kernel(const bf16_t* __restrict__ q_lat, const bf16_t* __restrict__ q_rows, const bf16_t* __restrict__ cache,
+                        const float* __restrict__ gate, const int32_t* __restrict__ block_tables, int max_blocks,
+                        const int64_t* __restrict__ positions, const int32_t* __restrict__ cu_q, int q_per_seq, int B, int H, int D,
+                        int R, int Cr, int block_size, int window, float scale, const float* __restrict__ freqs, float mag,
+                        int rot_dims, bf16_t* __restrict__ out) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
+  const int t = blockIdx.x, ht = blockIdx.y;
+  const int KW = Cr + R, KT = KW >> 5, CT_K = Cr >> 5, NT = Cr >> 4;
+  bf16_t* ct = reinterpret_cast<bf16_t*>(smem) + (size_t)wave * Cr * LAT_CTS;
+  int b;
+  if (cu_q) {
+    int lo = 0, hi = B;
+    while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (cu_q[mid] <= t) lo = mid; else hi = mid; }
+    b = lo;
+  } else {
+    b = t / q_per_seq;
+  }
+  const long p = positions[t];
+  const float pos = (float)p;
+  const long first = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int h = ht * 16 + i;
+  const bool hv = h < H;
+  // the head's query in the latent space | its rotated part, as B fragments: lane (head i, chunk g) holds k = kt * 32 + g * 8 .. + 7
+  u32x4_t qf[LAT_KT_MAX];
+  const bf16_t* ql = q_lat + ((size_t)t * H + (hv ? h : 0)) * Cr;
+  const bf16_t* qr = q_rows + ((size_t)t * H + (hv ? h : 0)) * (D + R) + D;
+#pragma unroll
+  for (int kt = 0; kt < LAT_KT_MAX; ++kt) {
+    qf[kt] = u32x4_t{0u, 0u, 0u, 0u};
+    if (kt < KT && hv) {
+      const int k = kt * 32 + g * 8;
+      if (k < Cr) {
+        qf[kt] = *reinterpret_cast<const u32x4_t*>(ql + k);
+      } else {
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = rope_entry([&](int j) { return bf2f(qr[j]); }, k - Cr + e, R, rot_dims, pos, freqs, mag);
+        qf[kt] = u32x4_t{pack_bf2(v[0], v[1]), pack_bf2(v[2], v[3]), pack_bf2(v[4], v[5]), pack_bf2(v[6], v[7])};
+      }
+    }
+  }
+  f32x4_t acc[LAT_NT_MAX];
+#pragma unroll
+  for (int nt = 0; nt < LAT_NT_MAX; ++nt) acc[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float mrun = -INFINITY, den = 0.f;
+  const int32_t* bt = block_tables + (size_t)b * max_blocks;
+  const int nsteps = (int)((p - first) >> 5) + 1;
+  const int slot0 = (i >> 2) * 8 + (i & 3);            // key (within the step) of A row i in the first tile; the second tile: + 4
+  for (int step = wave; step < nsteps; step += NW) {
+    const long j0 = first + (long)step * 32;
+    const long ja = j0 + slot0, jb = ja + 4;
+    const bool va = ja <= p, vb = jb <= p;
+    const bf16_t* ka = cache + (size_t)(va ? bt[ja / block_size] * block_size + (int)(ja % block_size) : 0) * KW + g * 8;
+    const bf16_t* kb = cache + (size_t)(vb ? bt[jb / block_size] * block_size + (int)(jb % block_size) : 0) * KW + g * 8;
+    f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    wave_sync();                                       // the previous step's readers of ct are done
+#pragma unroll
+    for (int kt = 0; kt < LAT_KT_MAX; ++kt) {
+      if (kt < KT) {
+        u32x4_t a0 = {0u, 0u, 0u, 0u}, a1 = {0u, 0u, 0u, 0u};
+        if (va) a0 = *reinterpret_cast<const u32x4_t*>(ka + kt * 32);
+        if (vb) a1 = *reinterpret_cast<const u32x4_t*>(kb + kt * 32);
+        s0 = mfma16(a0, qf[kt], s0);
+        s1 = mfma16(a1, qf[kt], s1);
+        if (kt < CT_K) {
+          bf16_t* c0 = ct + (size_t)(kt * 32 + g * 8) * LAT_CTS + slot0;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            c0[e * LAT_CTS] = (bf16_t)((a0[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+            c0[e * LAT_CTS + 4] = (bf16_t)((a1[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+          }
+        }
+      }
+    }
+    // lane (head i, g): keys j0 + g * 8 + 0 .. 7
+    float sv[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float raw = e < 4 ? s0[e] : s1[e - 4];
+      sv[e] = (j0 + g * 8 + e <= p) ? raw * scale : -INFINITY;
+      mx = fmaxf(mx, sv[e]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mn = fmaxf(mrun, mx);
+    const float resc = mrun == -INFINITY ? 0.f : expf(mrun - mn);
+    float ps = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { sv[e] = sv[e] == -INFINITY ? 0.f : expf(sv[e] - mn); ps += sv[e]; }
+    ps += __shfl_xor(ps, 16, 64);
+    ps += __shfl_xor(ps, 32, 64);
+    den = den * resc + ps;
+    mrun = mn;
+    const u32x4_t pb = {pack_bf2(sv[0], sv[1]), pack_bf2(sv[2], sv[3]), pack_bf2(sv[4], sv[5]), pack_bf2(sv[6], sv[7])};
+    wave_sync();                                       // ct is complete
+#pragma unroll
+    for (int nt = 0; nt < LAT_NT_MAX; ++nt) {
+      if (nt < NT) {
+        const u32x4_t a = *reinterpret_cast<const u32x4_t*>(ct + (size_t)(nt * 16 + i) * LAT_CTS + g * 8);
+        acc[nt] *= resc;
+        acc[nt] = mfma16(a, pb, acc[nt]);
+      }
+    }
+  }
+  // the waves' partial rows meet in LDS (each wave's own region, reused): [col][head] fp32, then m and den per head
+  wave_sync();
+  float* part = reinterpret_cast<float*>(ct);
+#pragma unroll
+  for (int nt = 0; nt < LAT_NT_MAX; ++nt)
+    if (nt < NT) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) part[(size_t)(nt * 16 + g * 4 + r) * 16 + i] = acc[nt][r];
+    }
+  if (g == 0) { part[(size_t)Cr * 16 + i] = mrun; part[(size_t)Cr * 16 + 16 + i] = den; }
+  __syncthreads();
+  const size_t wstride = (size_t)Cr * LAT_CTS / 2;      // floats per wave region
+  const float* all = reinterpret_cast<const float*>(smem);
+  float M = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) M = fmaxf(M, all[w * wstride + (size_t)Cr * 16 + i]);
+  float f[NW], Dn = 0.f;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) {
+    const float mw = all[w * wstride + (size_t)Cr * 16 + i];
+    f[w] = mw == -INFINITY ? 0.f : expf(mw - M);
+    Dn += all[w * wstride + (size_t)Cr * 16 + 16 + i] * f[w];
+  }
+  if (!hv) return;
+  const float gsc = gate[(size_t)t * H + h] / Dn;
+  for (int nt = wave; nt < NT; nt += NW) {
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float a = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) a += all[w * wstride + (size_t)(nt * 16 + g * 4 + r) * 16 + i] * f[w];
+      v[r] = a * gsc;
+    }
+    uint2 o2;
+    o2.x = pack_bf2(v[0], v[1]);
+    o2.y = pack_bf2(v[2], v[3]);
+    *reinterpret_cast<uint2*>(out + ((size_t)t * H + h) * Cr + nt * 16 + g * 4) = o2;
+  }
+}
+
+static inline bool latent_mfma_ok(int Cr, int R) {
+  return Cr % 32 == 0 && R % 32 == 0 && Cr <= 16 * LAT_NT_MAX && Cr + R <= 32 * LAT_KT_MAX;
+}
+
 }  // namespace
 
 #define LAUNCH_OK() (hipGetLastError() == hipSuccess ? SSD_OK : SSD_ERR_LAUNCH)
@@ -185,11 +354,33 @@ extern "C" int ssd_latent_store(const void* proj_rows, long ld, int q_rank, int 
 extern "C" int ssd_latent_attn(const void* q_abs, const void* q_rows, const void* cache, const void* gate, const int32_t* block_tables,
                                int max_blocks, const int64_t* positions, const int32_t* cu_q, int q_per_seq, int B, int T, int H, int D,
                                int rot, int kv_rank, int block_size, int window, float scale, const float* freqs, float mag,
-                               int rot_dims, void* out_rows, int f32, void* stream) {
+                               int rot_dims, void* out_rows, int f32, int q_abs_elem, void* stream) {
   if (!q_abs || !q_rows || !cache || !gate || !block_tables || !positions || !freqs || !out_rows) return SSD_ERR_ARG;
   if (B <= 0 || T <= 0 || H <= 0 || D <= 0 || rot < 0 || kv_rank <= 0 || kv_rank > 64 * LAT_MAXC || block_size <= 0 || max_blocks <= 0 ||
       rot_dims < 0 || rot_dims > rot || (rot_dims & 1) || (!cu_q && q_per_seq <= 0))
     return SSD_ERR_SHAPE;
+  if (q_abs_elem) {        // q_abs holds element-type rows: the MFMA form
+    if (f32 || !latent_mfma_ok(kv_rank, rot)) return SSD_ERR_SHAPE;
+    const dim3 mg(T, (H + 15) / 16);
+    if (kv_rank <= 256) {
+      const size_t mb = (size_t)4 * kv_rank * LAT_CTS * sizeof(bf16_t);
+      if (mb > 64 * 1024 && hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                (int)mb) != hipSuccess)
+        return SSD_ERR_LAUNCH;
+      hipLaunchKernelGGL(latent_attn_mfma_kernel<4>, mg, dim3(256), mb, (hipStream_t)stream, (const bf16_t*)q_abs, (const bf16_t*)q_rows,
+                         (const bf16_t*)cache, (const float*)gate, block_tables, max_blocks, positions, cu_q, q_per_seq, B, H, D, rot,
+                         kv_rank, block_size, window, scale, freqs, mag, rot_dims, (bf16_t*)out_rows);
+    } else {
+      const size_t mb = (size_t)2 * kv_rank * LAT_CTS * sizeof(bf16_t);
+      if (mb > 64 * 1024 && hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                (int)mb) != hipSuccess)
+        return SSD_ERR_LAUNCH;
+      hipLaunchKernelGGL(latent_attn_mfma_kernel<2>, mg, dim3(128), mb, (hipStream_t)stream, (const bf16_t*)q_abs, (const bf16_t*)q_rows,
+                         (const bf16_t*)cache, (const float*)gate, block_tables, max_blocks, positions, cu_q, q_per_seq, B, H, D, rot,
+                         kv_rank, block_size, window, scale, freqs, mag, rot_dims, (bf16_t*)out_rows);
+    }
+    return LAUNCH_OK();
+  }
   const size_t bytes = (size_t)4 * (kv_rank + rot + 128) * sizeof(float);
   const dim3 grid(T, (H + 3) / 4);
   if (f32)
@@ -201,4 +392,9 @@ extern "C" int ssd_latent_attn(const void* q_abs, const void* q_rows, const void
                        (const bf16_t*)q_rows, (const bf16_t*)cache, (const float*)gate, block_tables, max_blocks, positions, cu_q,
                        q_per_seq, B, H, D, rot, kv_rank, block_size, window, scale, freqs, mag, rot_dims, (bf16_t*)out_rows);
   return LAUNCH_OK();
+}
+
+extern "C" int ssd_latent_attn_mfma_ok(int kv_rank, int rot, int f32) {
+  if (kv_rank <= 0 || rot < 0) return SSD_ERR_SHAPE;
+  return (!f32 && latent_mfma_ok(kv_rank, rot)) ? 1 : 0;
 }

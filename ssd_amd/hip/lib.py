@@ -136,7 +136,8 @@ SIGNATURES = {
     "ssd_latent_store": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_float, c_int,
                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "ssd_latent_attn": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                        c_int, c_int, c_int, c_int, c_float, c_void_p, c_float, c_int, c_void_p, c_int, c_void_p],
+                        c_int, c_int, c_int, c_int, c_float, c_void_p, c_float, c_int, c_void_p, c_int, c_int, c_void_p],
+    "ssd_latent_attn_mfma_ok": [c_int, c_int, c_int],
     "ssd_lightning_scan": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                            c_int, c_int, c_int, c_int, c_void_p],
     "ssd_lightning_gate_norm": [c_void_p, c_void_p, c_long, c_int, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -188,6 +189,9 @@ def load_library(family: str | None = None):
     global _LIB
     if _LIB is not None:
         return _LIB
+    # PyTorch ships its own HIP runtime; it has to be in the process BEFORE this library is opened, or the library binds the system's
+    # copy and its kernels live in another runtime than torch's streams and allocations (every launch then fails)
+    import torch  # noqa: F401
     path, partial = lib_path(), False
     if not os.path.exists(path) and family in FAMILY_SOURCES and os.path.exists(family_lib_path(family)):
         path, partial = family_lib_path(family), True

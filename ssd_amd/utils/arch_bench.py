@@ -1,8 +1,13 @@
-"""bench.py --workload fatulix: prefill and decode throughput of the Fatulix decoder at layer sizes that resemble real models (random
+"""bench.py --workload fatulix | zerusun: prefill and decode throughput of the Fatulix decoder at layer sizes that resemble real models (random
 weights), beside the closest existing family -- a dense grouped-query Llama decoder -- at equal active size: the same width, query /
 key / value / output projection sizes (two 64-wide maps per head = one 128-wide head), the same feed-forward parameters per token
 (top * 2 * ff + 2 * shared_ff = 3 * intermediate), layers, vocabulary, prompt and batch.  Both run through the same ModelRunner paths
-(`run(seqs, is_prefill)`: staging, varlen prefill / hipGraph decode, LM head, argmax)."""
+(`run(seqs, is_prefill)`: staging, varlen prefill / hipGraph decode, LM head, argmax).
+
+--workload zerusun: the Zerusun decoder (layers alternate latent attention with a sliding window and linear attention over a recurrent
+state; routed three-matrix experts with group-limited choice and a gated shared expert; the stack is one loop of one pass) beside
+the closest existing family, Fatulix, at equal size: the same width, layers, vocabulary, experts, top and feed-forward parameters per
+token (three-matrix experts of 2/3 the two-matrix experts' ff), mixers of about the same parameter count."""
 from __future__ import annotations
 
 import json
@@ -13,7 +18,8 @@ import torch
 from ssd_amd.config import Config
 from ssd_amd.engine.block_manager import BlockManager
 from ssd_amd.engine.sequence import Sequence
-from ssd_amd.model_config import DiffAttention, FatulixConfig, FatulixLayer, ModelConfig, RoutedMLP
+from ssd_amd.model_config import (DiffAttention, FatulixConfig, FatulixLayer, GroupRoutedMLP, LatentAttention, LightningAttention, ModelConfig,
+                                  RopeSpec, RoutedMLP, ZerusunConfig, ZerusunLayer)
 
 VOCAB = 32000
 SIZES = {
@@ -32,6 +38,18 @@ def models(size: str):
     return fat, llama
 
 
+def zerusun_models(size: str):
+    """(Zerusun, Fatulix) of equal size."""
+    W, L, Hh, G, E, top, ff, sff, inter = SIZES[size]
+    fat, _ = models(size)
+    rope = RopeSpec(64, 1e6, {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0})
+    mlp = GroupRoutedMLP(E, top, ff * 2 // 3, 4, 2, 1.5, sff * 2 // 3)
+    lat = ZerusunLayer(LatentAttention(Hh, 128, 64, 128, 3 * W // 8, 512, 192 ** -0.5, 1024, rope), mlp)
+    lin = ZerusunLayer(LightningAttention(Hh // 2, 128, 128, [1.0 - 2.0 ** -(3 + 5 * h / (Hh // 2)) for h in range(Hh // 2)]), mlp)
+    zer = ZerusunConfig(VOCAB, W, 1e-5, [lat, lin] * (L // 2), 0, L, 1)
+    return zer, fat
+
+
 def _runner(cfg, max_len: int, batch: int, dtype: str = "bfloat16"):
     from ssd_amd.engine.model_runner import ModelRunner
     bs = 256
@@ -40,7 +58,8 @@ def _runner(cfg, max_len: int, batch: int, dtype: str = "bfloat16"):
                     max_num_batched_tokens=max(max_len, 4096), num_kvcache_blocks=blocks)
     Sequence.block_size = bs
     runner = ModelRunner(config, cfg, is_draft=False, device=torch.device("cuda", 0), weights_seed=0, num_kvcache_blocks=blocks)
-    return runner, BlockManager(blocks, bs, max_model_len=max_len, prefix_cache=False)
+    return runner, BlockManager(blocks, bs, max_model_len=max_len, prefix_cache=False,
+                                state_slots=batch if getattr(cfg, "recurrent", False) else 0)
 
 
 def _timed(fn, steps: int, warmup: int) -> float:
@@ -98,6 +117,35 @@ def measure(cfg, prompt_len: int, batch: int, steps: int, warmup: int) -> dict:
     del runner
     torch.cuda.empty_cache()
     return out
+
+
+def run_zerusun(args) -> dict:
+    steps, warmup = args.steps, args.warmup
+    prompt_len = args.input_len if args.input_len != 128 else 2048
+    results = {}
+    sizes = list(SIZES) if getattr(args, "arch_size", "all") == "all" else [args.arch_size]
+    batches = (1, 8) if not getattr(args, "arch_batch", 0) else (args.arch_batch,)
+    only = getattr(args, "arch_only", "both")
+    for size in sizes:
+        zer, fat = zerusun_models(size)
+        for batch in batches:
+            key = f"{size} prompt={prompt_len} batch={batch}"
+            results[key] = {}
+            if only in ("both", "zerusun"):
+                results[key]["zerusun"] = measure(zer, prompt_len, batch, steps, warmup)
+            if only in ("both", "fatulix"):
+                results[key]["fatulix_equal_size"] = measure(fat, prompt_len, batch, steps, warmup)
+            print(f"[arch_bench] {key}: {json.dumps(results[key])}", flush=True)
+    k = f"w4096 prompt={prompt_len} batch=8"
+    if k not in results or len(results[k]) < 2:
+        return {"metric": "Zerusun / equal-size Fatulix throughput (partial run)", "sizes": results}
+    return {"metric": "decode tokens/s, Zerusun w4096 (4 layers: latent attention / linear attention, 16 experts top 2 + shared), batch 8, "
+                      "beside an equal-size Fatulix decoder",
+            "value": results[k]["zerusun"]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": results[k]["zerusun"]["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic (random weights, random tokens)",
+            "config": {"model": "zerusun-w4096-synthetic", "global_batch": 8, "seq_len": prompt_len, "parallelism": "single GPU"},
+            "closest_model_value": results[k]["fatulix_equal_size"]["decode_tok_s"], "sizes": results}
 
 
 def run(args) -> dict:

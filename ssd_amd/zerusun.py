@@ -73,7 +73,10 @@ class HipZerusun(Res32Decoder):
         if lat:
             self.cq = z(T * max(m.q_rank for m in lat), dtype=el)
             self.q = z(T * max(m.heads * (m.dim + m.rot_dim) for m in lat), dtype=el)
-            self.q_abs = z(T * max(m.heads * m.kv_rank for m in lat))
+            self.q_abs = z(T * max(m.heads * m.kv_rank for m in lat))           # queries in the latent space: fp32, or (its first half)
+            self.q_lat = self.q_abs.view(el)                                     # element-type rows where the MFMA attention takes them
+            self.mfma = {i: H.latent_attn_mfma_ok(l.mixer.kv_rank, l.mixer.rot_dim, self.f32) for i, l in enumerate(cfg.layers)
+                         if l.mixer.kind == "latent_attention"}
             self.gate = z(T * max(m.heads for m in lat))
             self.olat = z(T * max(m.heads * m.kv_rank for m in lat), dtype=el)
         if lin:
@@ -219,9 +222,12 @@ class HipZerusun(Res32Decoder):
             H.latent_store(self.proj, NP, m.q_rank, Cr, R, Hh, w[p + "dq.norm"], w[p + "dkv.norm"], cfg.rms_norm_eps, positions, freqs,
                            mag, m.rope.dims, meta.slot_mapping, self.cq, self.kv[run], self.gate, T, f)
             H.gemm_rows(self.cq, w[p + "uq"], self.q, T, Hh * (D + R), m.q_rank, f, H.GR_ELEM)
-            H.gemm_rows_batched(self.q, w[p + "ukt"], self.q_abs, T, Cr, D, Hh, Hh * (D + R), D + R, Hh * Cr, Cr, f)
-            H.latent_attn(self.q_abs, self.q, self.kv[run], self.gate, meta.block_tables, self.max_blocks, positions, meta.B, T, Hh, D,
-                          R, Cr, self.block_size, m.window, m.scale, freqs, mag, m.rope.dims, self.olat, f, **seqs)
+            mf = self.mfma[li]
+            H.gemm_rows_batched(self.q, w[p + "ukt"], self.q_lat if mf else self.q_abs, T, Cr, D, Hh, Hh * (D + R), D + R, Hh * Cr, Cr, f,
+                                H.GR_ELEM if mf else H.GR_F32)
+            H.latent_attn(self.q_lat if mf else self.q_abs, self.q, self.kv[run], self.gate, meta.block_tables, self.max_blocks, positions,
+                          meta.B, T, Hh, D, R, Cr, self.block_size, m.window, m.scale, freqs, mag, m.rope.dims, self.olat, f,
+                          q_abs_elem=mf, **seqs)
             H.gemm_rows_batched(self.olat, w[p + "uv"], self.att, T, m.vdim, Cr, Hh, Hh * Cr, Cr, Hh * m.vdim, m.vdim, f, H.GR_ELEM)
         else:
             Hh, D, Dv = m.heads, m.dim, m.vdim

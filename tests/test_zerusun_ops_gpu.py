@@ -117,9 +117,11 @@ def _pages(n_seq, lens, bs, seed):
 
 @pytest.mark.parametrize("f32", [True, False])
 @pytest.mark.parametrize("Hh,D,R,Cr,Qr,win,rd,bs", [(6, 32, 32, 128, 64, 40, 32, 64), (3, 8, 6, 20, 12, 5, 4, 16), (5, 16, 8, 72, 40, 0, 8, 16),
-                                                    (1, 8, 2, 8, 8, 1, 2, 16)])
+                                                    (1, 8, 2, 8, 8, 1, 2, 16), (20, 16, 64, 512, 32, 33, 48, 16), (17, 8, 32, 32, 16, 0, 32, 32),
+                                                    (16, 8, 32, 288, 16, 32, 2, 16)])
 def test_latent_store_and_windowed_attention_over_scattered_pages(f32, Hh, D, R, Cr, Qr, win, rd, bs):
-    """Two sequences; the second arrives in two launches (a portion, then the rest) and must see the keys of the first launch."""
+    """Two sequences; the second arrives in two launches (a portion, then the rest) and must see the keys of the first launch.  Where the
+    MFMA form takes the sizes (bf16, latent sizes in multiples of 32) it is the one that runs, with the latent-space queries as bf16 rows."""
     el = elem(f32)
     lens = [37, 50]
     eps, scale = 1e-5, 0.2
@@ -133,6 +135,10 @@ def test_latent_store_and_windowed_attention_over_scattered_pages(f32, Hh, D, R,
     proj_all = [rnd(n, NP, seed=10 + i) for i, n in enumerate(lens)]
     q_all = [rnd(n, Hh * (D + R), seed=20 + i).to(el) for i, n in enumerate(lens)]
     qabs_all = [rnd(n, Hh * Cr, seed=30 + i) for i, n in enumerate(lens)]
+    mfma = H().latent_attn_mfma_ok(Cr, R, f32)
+    assert mfma == ((not f32) and Cr % 32 == 0 and R % 32 == 0)
+    if mfma:
+        qabs_all = [q.bfloat16() for q in qabs_all]
 
     def launch(parts):
         """parts: [(seq, lo, hi)] -> out rows of all parts."""
@@ -148,7 +154,7 @@ def test_latent_store_and_windowed_attention_over_scattered_pages(f32, Hh, D, R,
         out = torch.zeros(T, Hh * Cr, dtype=el, device=DEV)
         tables = torch.stack([bt[s] for s, _, _ in parts])
         H().latent_attn(d(qa), d(q), cache, gate, d(tables), mb, d(pos), len(parts), T, Hh, D, R, Cr, bs, win, scale, d(fq), mag, rd, out,
-                        f32, cu_q=d(cu))
+                        f32, cu_q=d(cu), q_abs_elem=mfma)
         return cq, out
 
     cq1, o1 = launch([(0, 0, 37), (1, 0, 21)])

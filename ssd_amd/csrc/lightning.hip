@@ -6,6 +6,7 @@
 // writes the slot back, so a prompt may arrive in portions of any size and decoding is the one-row case of the same kernel.
 //  * ssd_lightning_scan       proj rows fp32 [T][ld] holding [q | k | v | ...] -> o fp32 [T][H*Dv], state updated in place
 //  * ssd_lightning_gate_norm  out = w * o / sqrt(mean(o^2) + eps) * sigmoid(g) over the concatenated heads, as GEMM-input rows
+// Two forms: state in registers (usual head sizes; below) and state in LDS (any sizes).
 // The arithmetic of a row is the same whatever the portion: per state element one multiply-add chain in token order, the output a sum
 // over d in a fixed order -- whole prompt, portions and token-by-token decoding give bit-identical rows.
 #include "common.h"
@@ -75,6 +76,66 @@ lightning_scan_kernel(const float* __restrict__ proj, long ld, int q_off, int k_
   for (int i = tid; i < D * Dv; i += 256) sp[i] = S[i];
 }
 
+// Register form (D = 8 * EPT with EPT in {4, 8, 16, 32}, Dv % 32 == 0): a workgroup owns 32 state columns of one (sequence, head) --
+// grid.z walks the column blocks -- and thread (g, e) keeps the EPT elements (d = g + 8 n, column e) in registers.  Rows are staged
+// eight at a time (silu applied once), every thread then walks the eight tokens without a barrier (it touches only its own state and
+// the staged rows), and the eight d-groups' partial outputs are summed in group order.  The arithmetic of a row is the same for any
+// portioning: the per-element chain in token order, the output sum over n ascending, then over g ascending.
+template <int EPT>
+__global__ void __launch_bounds__(256)
+lightning_scan_reg_kernel(const float* __restrict__ proj, long ld, int q_off, int k_off, int v_off, const float* __restrict__ decay,
+                          const int64_t* __restrict__ positions, const int32_t* __restrict__ cu_q, int q_per_seq,
+                          const int32_t* __restrict__ state_slots, float* __restrict__ state, float* __restrict__ out, int H, int Dv) {
+  constexpr int TB = 8, NG = 8, CB = 32, D = NG * EPT;
+  __shared__ float sq[TB][D], sk[TB][D];
+  __shared__ float sv[TB][CB];
+  __shared__ float po[TB][NG][CB];
+  const int b = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * CB, tid = threadIdx.x;
+  const int g = tid >> 5, e = tid & 31;
+  const int row0 = cu_q ? cu_q[b] : b * q_per_seq;
+  const int row1 = cu_q ? cu_q[b + 1] : (b + 1) * q_per_seq;
+  if (row1 <= row0) return;
+  float* sp = state + ((size_t)state_slots[b] * H + h) * D * Dv + c0 + e;
+  const bool fresh = positions[row0] == 0;
+  float S[EPT];
+#pragma unroll
+  for (int n = 0; n < EPT; ++n) S[n] = fresh ? 0.f : sp[(size_t)(g + NG * n) * Dv];
+  const float dc = decay[h];
+  for (int r = row0; r < row1; r += TB) {
+    const int nb = row1 - r < TB ? row1 - r : TB;
+    __syncthreads();                      // the previous batch's readers are done
+    for (int idx = tid; idx < nb * D; idx += 256) {
+      const int tt = idx / D, d = idx % D;
+      const float* pr = proj + (size_t)(r + tt) * ld + h * D + d;
+      sq[tt][d] = siluf_(pr[q_off]);
+      sk[tt][d] = siluf_(pr[k_off]);
+    }
+    if (tid < nb * CB) sv[tid >> 5][tid & 31] = siluf_(proj[(size_t)(r + (tid >> 5)) * ld + v_off + h * Dv + c0 + (tid & 31)]);
+    __syncthreads();
+    for (int tt = 0; tt < nb; ++tt) {
+      const float ve = sv[tt][e];
+      float o = 0.f;
+#pragma unroll
+      for (int n = 0; n < EPT; ++n) {
+        const int d = g + NG * n;
+        const float s = fmaf(dc, S[n], sk[tt][d] * ve);
+        S[n] = s;
+        o = fmaf(s, sq[tt][d], o);
+      }
+      po[tt][g][e] = o;
+    }
+    __syncthreads();
+    if (g < nb) {                         // thread (g, e) now finishes token g of the batch
+      float o = 0.f;
+#pragma unroll
+      for (int gg = 0; gg < NG; ++gg) o += po[g][gg][e];
+      out[(size_t)(r + g) * H * Dv + h * Dv + c0 + e] = o;
+    }
+  }
+#pragma unroll
+  for (int n = 0; n < EPT; ++n) sp[(size_t)(g + NG * n) * Dv] = S[n];
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 lightning_gate_norm_kernel(const float* __restrict__ o, const float* __restrict__ proj, long ld, int g_off, const T* __restrict__ w,
@@ -102,6 +163,18 @@ extern "C" int ssd_lightning_scan(const void* proj_rows, long ld, int q_off, int
                                   void* state, void* out_rows, int B, int H, int D, int Dv, void* stream) {
   if (!proj_rows || !decay || !positions || !state_slots || !state || !out_rows) return SSD_ERR_ARG;
   if (B <= 0 || H <= 0 || D <= 0 || Dv <= 0 || (!cu_q && q_per_seq <= 0)) return SSD_ERR_SHAPE;
+  if (Dv % 32 == 0 && Dv / 32 <= 65535 && (D == 32 || D == 64 || D == 128 || D == 256)) {
+    const dim3 grid(B, H, Dv / 32);
+#define SCAN_REG(EPT)                                                                                                              \
+  hipLaunchKernelGGL(lightning_scan_reg_kernel<EPT>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)proj_rows, ld, q_off,  \
+                     k_off, v_off, decay, positions, cu_q, q_per_seq, state_slots, (float*)state, (float*)out_rows, H, Dv)
+    if (D == 32) SCAN_REG(4);
+    else if (D == 64) SCAN_REG(8);
+    else if (D == 128) SCAN_REG(16);
+    else SCAN_REG(32);
+#undef SCAN_REG
+    return LAUNCH_OK();
+  }
   int EP = 1;
   while (EP < Dv && EP < 256) EP <<= 1;
   const size_t bytes = ((size_t)D * Dv + 2 * (size_t)D + Dv + (size_t)(256 / EP) * Dv) * sizeof(float);

@@ -178,9 +178,10 @@ def test_latent_store_and_windowed_attention_over_scattered_pages(f32, Hh, D, R,
     assert torch.allclose(cq1[:37].cpu().double(), ref_cq, **tol(f32))
 
 
-@pytest.mark.parametrize("Hh,D,Dv", [(6, 32, 32), (3, 16, 24), (1, 8, 1), (2, 40, 130), (2, 128, 128)])
+@pytest.mark.parametrize("Hh,D,Dv", [(6, 32, 32), (3, 16, 24), (1, 8, 1), (2, 40, 130), (2, 128, 128), (3, 64, 96), (1, 256, 32), (2, 32, 48)])
 def test_lightning_scan_in_portions_over_state_slots(Hh, D, Dv):
-    """Three sequences over four slots (filled with NaN: a sequence that starts at position 0 must not read its slot), fed whole, in
+    """Head sizes of the register form (dim 32 / 64 / 128 / 256, vdim in multiples of 32) and of the LDS form (anything else).
+    Three sequences over four slots (filled with NaN: a sequence that starts at position 0 must not read its slot), fed whole, in
     portions and token by token; the state of a portion's end is what the next portion starts from."""
     lens = [29, 1, 14]
     decay = torch.tensor([math.exp(-1.0 / (1.5 ** (h + 1))) for h in range(Hh)])

@@ -458,11 +458,12 @@ int ssd_latent_store(const void* proj_rows, long ld, int q_rank, int kv_rank, in
                      const int32_t* slots, void* cq_out, void* cache, void* gate_out, int T, int f32, void* stream);
 /* out[t][h] (kv_rank wide) = gate[t][h] * sum_j softmax_j(scale * (<q_abs[t][h], c_j> + <rope(q_rows[t][h][D:]), k_j>)) c_j over the
  * keys j of the token's sequence with 0 <= positions[t] - j < window (window <= 0: all keys up to the token); q_abs fp32
- * [T][H][kv_rank] (element-type rows when q_abs_elem), q_rows [T][H][D + rot].  Sequences: cu_q int32 [B+1] row ranges, or q_per_seq rows each when cu_q is NULL. */
+ * [T][H][kv_rank] (element-type rows when q_abs_elem), q_rows [T][H][D + rot].  workspace (optional, fp32): with few rows the MFMA
+ * form cuts the window over up to 16 workgroups per (token, 16 heads), kv_rank * 16 + 32 floats per slice, and merges.  Sequences: cu_q int32 [B+1] row ranges, or q_per_seq rows each when cu_q is NULL. */
 int ssd_latent_attn(const void* q_abs, const void* q_rows, const void* cache, const void* gate, const int32_t* block_tables,
                     int max_blocks, const int64_t* positions, const int32_t* cu_q, int q_per_seq, int B, int T, int H, int D, int rot,
                     int kv_rank, int block_size, int window, float scale, const float* freqs, float mag, int rot_dims, void* out_rows,
-                    int f32, int q_abs_elem, void* stream);
+                    int f32, int q_abs_elem, void* workspace, long workspace_bytes, void* stream);
 /* 1 when the MFMA form of ssd_latent_attn takes these sizes (then the caller may hand q_abs over as element-type rows, q_abs_elem = 1:
  * 16 heads of a token per workgroup, keys in steps of 32), 0 when only the scalar form (fp32 q_abs, q_abs_elem = 0) does. */
 int ssd_latent_attn_mfma_ok(int kv_rank, int rot, int f32);

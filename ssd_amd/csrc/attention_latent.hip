@@ -181,7 +181,7 @@ latent_attn_mfma_kernel(const bf16_t* __restrict__ q_lat, const bf16_t* __restri
                         const float* __restrict__ gate, const int32_t* __restrict__ block_tables, int max_blocks,
                         const int64_t* __restrict__ positions, const int32_t* __restrict__ cu_q, int q_per_seq, int B, int H, int D,
                         int R, int Cr, int block_size, int window, float scale, const float* __restrict__ freqs, float mag,
-                        int rot_dims, bf16_t* __restrict__ out) {
+                        int rot_dims, bf16_t* __restrict__ out, int ksplit, float* __restrict__ ws) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
   const int t = blockIdx.x, ht = blockIdx.y;
@@ -226,7 +226,7 @@ latent_attn_mfma_kernel(const bf16_t* __restrict__ q_lat, const bf16_t* __restri
   const int32_t* bt = block_tables + (size_t)b * max_blocks;
   const int nsteps = (int)((p - first) >> 5) + 1;
   const int slot0 = (i >> 2) * 8 + (i & 3);            // key (within the step) of A row i in the first tile; the second tile: + 4
-  for (int step = wave; step < nsteps; step += NW) {
+  for (int step = blockIdx.z * NW + wave; step < nsteps; step += NW * ksplit) {
     const long j0 = first + (long)step * 32;
     const long ja = j0 + slot0, jb = ja + 4;
     const bool va = ja <= p, vb = jb <= p;
@@ -306,6 +306,19 @@ latent_attn_mfma_kernel(const bf16_t* __restrict__ q_lat, const bf16_t* __restri
     f[w] = mw == -INFINITY ? 0.f : expf(mw - M);
     Dn += all[w * wstride + (size_t)Cr * 16 + 16 + i] * f[w];
   }
+  if (ksplit > 1) {        // few rows: the window is cut over ksplit workgroups; this one's sums (relative to its M) go to the workspace
+    float* u = ws + ((size_t)(t * gridDim.y + ht) * ksplit + blockIdx.z) * ((size_t)Cr * 16 + 32);
+    if (wave == 0 && g == 0) { u[(size_t)Cr * 16 + i] = M; u[(size_t)Cr * 16 + 16 + i] = Dn; }
+    for (int nt = wave; nt < NT; nt += NW)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float a = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) a += all[w * wstride + (size_t)(nt * 16 + g * 4 + r) * 16 + i] * f[w];
+        u[(size_t)(nt * 16 + g * 4 + r) * 16 + i] = a;
+      }
+    return;
+  }
   if (!hv) return;
   const float gsc = gate[(size_t)t * H + h] / Dn;
   for (int nt = wave; nt < NT; nt += NW) {
@@ -322,6 +335,28 @@ latent_attn_mfma_kernel(const bf16_t* __restrict__ q_lat, const bf16_t* __restri
     o2.y = pack_bf2(v[2], v[3]);
     *reinterpret_cast<uint2*>(out + ((size_t)t * H + h) * Cr + nt * 16 + g * 4) = o2;
   }
+}
+
+// The key slices of a row meet: out = gate * sum_z vals_z e^(M_z - M) / sum_z den_z e^(M_z - M), slices in order.
+__global__ void __launch_bounds__(256)
+latent_attn_merge_kernel(const float* __restrict__ ws, const float* __restrict__ gate, int H, int Cr, int HT, int ksplit,
+                         bf16_t* __restrict__ out) {
+  // a workgroup: 16 latent columns x 16 heads of one (token, head tile); thread = one output element
+  const int t = blockIdx.x / HT, ht = blockIdx.x % HT;
+  const size_t unit = (size_t)Cr * 16 + 32;
+  const float* u = ws + (size_t)blockIdx.x * ksplit * unit;
+  const int idx = blockIdx.y * 256 + threadIdx.x, i = idx & 15, col = idx >> 4, h = ht * 16 + i;
+  if (col >= Cr || h >= H) return;
+  float M = -INFINITY;
+  for (int z = 0; z < ksplit; ++z) M = fmaxf(M, u[z * unit + (size_t)Cr * 16 + i]);
+  float Dn = 0.f, a = 0.f;
+  for (int z = 0; z < ksplit; ++z) {
+    const float mz = u[z * unit + (size_t)Cr * 16 + i];
+    const float fz = mz == -INFINITY ? 0.f : expf(mz - M);
+    Dn += u[z * unit + (size_t)Cr * 16 + 16 + i] * fz;
+    a += u[z * unit + idx] * fz;
+  }
+  out[((size_t)t * H + h) * Cr + col] = (bf16_t)f2bf(a * (gate[(size_t)t * H + h] / Dn));
 }
 
 static inline bool latent_mfma_ok(int Cr, int R) {
@@ -354,14 +389,27 @@ extern "C" int ssd_latent_store(const void* proj_rows, long ld, int q_rank, int 
 extern "C" int ssd_latent_attn(const void* q_abs, const void* q_rows, const void* cache, const void* gate, const int32_t* block_tables,
                                int max_blocks, const int64_t* positions, const int32_t* cu_q, int q_per_seq, int B, int T, int H, int D,
                                int rot, int kv_rank, int block_size, int window, float scale, const float* freqs, float mag,
-                               int rot_dims, void* out_rows, int f32, int q_abs_elem, void* stream) {
+                               int rot_dims, void* out_rows, int f32, int q_abs_elem, void* workspace, long workspace_bytes,
+                               void* stream) {
   if (!q_abs || !q_rows || !cache || !gate || !block_tables || !positions || !freqs || !out_rows) return SSD_ERR_ARG;
   if (B <= 0 || T <= 0 || H <= 0 || D <= 0 || rot < 0 || kv_rank <= 0 || kv_rank > 64 * LAT_MAXC || block_size <= 0 || max_blocks <= 0 ||
       rot_dims < 0 || rot_dims > rot || (rot_dims & 1) || (!cu_q && q_per_seq <= 0))
     return SSD_ERR_SHAPE;
   if (q_abs_elem) {        // q_abs holds element-type rows: the MFMA form
     if (f32 || !latent_mfma_ok(kv_rank, rot)) return SSD_ERR_SHAPE;
-    const dim3 mg(T, (H + 15) / 16);
+    const int HT = (H + 15) / 16, NWv = kv_rank <= 256 ? 4 : 2;
+    // few rows (decoding): cut the window over up to 16 workgroups per (token, 16 heads) and merge; the cut depends on T alone
+    int ksplit = 1;
+    const long unit_bytes = ((long)kv_rank * 16 + 32) * (long)sizeof(float);
+    if (workspace && (long)T * HT < 256) {
+      const int steps = window > 0 ? (window + 31) / 32 + 1 : 64;
+      ksplit = 512 / (T * HT);
+      if (ksplit > (steps + NWv - 1) / NWv) ksplit = (steps + NWv - 1) / NWv;
+      if (ksplit > 16) ksplit = 16;
+      while (ksplit > 1 && (long)T * HT * ksplit * unit_bytes > workspace_bytes) --ksplit;
+      if (ksplit < 1) ksplit = 1;
+    }
+    const dim3 mg(T, HT, ksplit);
     if (kv_rank <= 256) {
       const size_t mb = (size_t)4 * kv_rank * LAT_CTS * sizeof(bf16_t);
       if (mb > 64 * 1024 && hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -369,7 +417,7 @@ extern "C" int ssd_latent_attn(const void* q_abs, const void* q_rows, const void
         return SSD_ERR_LAUNCH;
       hipLaunchKernelGGL(latent_attn_mfma_kernel<4>, mg, dim3(256), mb, (hipStream_t)stream, (const bf16_t*)q_abs, (const bf16_t*)q_rows,
                          (const bf16_t*)cache, (const float*)gate, block_tables, max_blocks, positions, cu_q, q_per_seq, B, H, D, rot,
-                         kv_rank, block_size, window, scale, freqs, mag, rot_dims, (bf16_t*)out_rows);
+                         kv_rank, block_size, window, scale, freqs, mag, rot_dims, (bf16_t*)out_rows, ksplit, (float*)workspace);
     } else {
       const size_t mb = (size_t)2 * kv_rank * LAT_CTS * sizeof(bf16_t);
       if (mb > 64 * 1024 && hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -377,8 +425,11 @@ extern "C" int ssd_latent_attn(const void* q_abs, const void* q_rows, const void
         return SSD_ERR_LAUNCH;
       hipLaunchKernelGGL(latent_attn_mfma_kernel<2>, mg, dim3(128), mb, (hipStream_t)stream, (const bf16_t*)q_abs, (const bf16_t*)q_rows,
                          (const bf16_t*)cache, (const float*)gate, block_tables, max_blocks, positions, cu_q, q_per_seq, B, H, D, rot,
-                         kv_rank, block_size, window, scale, freqs, mag, rot_dims, (bf16_t*)out_rows);
+                         kv_rank, block_size, window, scale, freqs, mag, rot_dims, (bf16_t*)out_rows, ksplit, (float*)workspace);
     }
+    if (ksplit > 1)
+      hipLaunchKernelGGL(latent_attn_merge_kernel, dim3(T * HT, (kv_rank + 15) / 16), dim3(256), 0, (hipStream_t)stream,
+                         (const float*)workspace, (const float*)gate, H, kv_rank, HT, ksplit, (bf16_t*)out_rows);
     return LAUNCH_OK();
   }
   const size_t bytes = (size_t)4 * (kv_rank + rot + 128) * sizeof(float);

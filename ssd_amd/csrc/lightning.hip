@@ -101,17 +101,37 @@ lightning_scan_reg_kernel(const float* __restrict__ proj, long ld, int q_off, in
 #pragma unroll
   for (int n = 0; n < EPT; ++n) S[n] = fresh ? 0.f : sp[(size_t)(g + NG * n) * Dv];
   const float dc = decay[h];
+  // raw projection values of the next batch travel in registers while the current batch is computed (a batch is short: without
+  // this every batch would wait a full memory round trip)
+  constexpr int QK = TB * D / 256;         // q / k elements of a batch per thread
+  float rq[QK], rk[QK], rv = 0.f;
+  auto fetch = [&](int r) {
+    const int nb = row1 - r < TB ? row1 - r : TB;
+#pragma unroll
+    for (int c = 0; c < QK; ++c) {
+      const int idx = tid + 256 * c, tt = idx / D, d = idx % D;
+      rq[c] = rk[c] = 0.f;
+      if (tt < nb) {
+        const float* pr = proj + (size_t)(r + tt) * ld + h * D + d;
+        rq[c] = pr[q_off];
+        rk[c] = pr[k_off];
+      }
+    }
+    rv = g < nb ? proj[(size_t)(r + g) * ld + v_off + h * Dv + c0 + e] : 0.f;
+  };
+  fetch(row0);
   for (int r = row0; r < row1; r += TB) {
     const int nb = row1 - r < TB ? row1 - r : TB;
     __syncthreads();                      // the previous batch's readers are done
-    for (int idx = tid; idx < nb * D; idx += 256) {
-      const int tt = idx / D, d = idx % D;
-      const float* pr = proj + (size_t)(r + tt) * ld + h * D + d;
-      sq[tt][d] = siluf_(pr[q_off]);
-      sk[tt][d] = siluf_(pr[k_off]);
+#pragma unroll
+    for (int c = 0; c < QK; ++c) {
+      const int idx = tid + 256 * c;
+      sq[idx / D][idx % D] = siluf_(rq[c]);
+      sk[idx / D][idx % D] = siluf_(rk[c]);
     }
-    if (tid < nb * CB) sv[tid >> 5][tid & 31] = siluf_(proj[(size_t)(r + (tid >> 5)) * ld + v_off + h * Dv + c0 + (tid & 31)]);
+    sv[g][e] = siluf_(rv);
     __syncthreads();
+    if (r + TB < row1) fetch(r + TB);
     for (int tt = 0; tt < nb; ++tt) {
       const float ve = sv[tt][e];
       float o = 0.f;

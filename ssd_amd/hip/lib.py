@@ -136,7 +136,7 @@ SIGNATURES = {
     "ssd_latent_store": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_float, c_int,
                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "ssd_latent_attn": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                        c_int, c_int, c_int, c_int, c_float, c_void_p, c_float, c_int, c_void_p, c_int, c_int, c_void_p],
+                        c_int, c_int, c_int, c_int, c_float, c_void_p, c_float, c_int, c_void_p, c_int, c_int, c_void_p, c_long, c_void_p],
     "ssd_latent_attn_mfma_ok": [c_int, c_int, c_int],
     "ssd_lightning_scan": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                            c_int, c_int, c_int, c_int, c_void_p],

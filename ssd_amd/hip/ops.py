@@ -492,11 +492,13 @@ def latent_store(proj, ld: int, q_rank: int, kv_rank: int, rot: int, H: int, q_n
 
 def latent_attn(q_abs, q_rows, cache, gate, block_tables, max_blocks: int, positions, B: int, T: int, H: int, D: int, rot: int,
                 kv_rank: int, block_size: int, window: int, scale: float, freqs, mag: float, rot_dims: int, out_rows, f32: bool,
-                cu_q=None, q_per_seq: int = 0, q_abs_elem: bool = False):
+                cu_q=None, q_per_seq: int = 0, q_abs_elem: bool = False, workspace=None):
     """q_abs_elem: q_abs holds element-type rows and the MFMA form runs (latent_attn_mfma_ok says whether it takes the sizes)."""
     _check(load_library().ssd_latent_attn(_p(q_abs), _p(q_rows), _p(cache), _p(gate), _p(block_tables), max_blocks, _p(positions),
                                           _p(cu_q), q_per_seq, B, T, H, D, rot, kv_rank, block_size, window, scale, _p(freqs), mag,
-                                          rot_dims, _p(out_rows), int(f32), int(q_abs_elem), _stream()), "ssd_latent_attn")
+                                          rot_dims, _p(out_rows), int(f32), int(q_abs_elem), _p(workspace),
+                                          workspace.numel() * workspace.element_size() if workspace is not None else 0, _stream()),
+           "ssd_latent_attn")
 
 
 def latent_attn_mfma_ok(kv_rank: int, rot: int, f32: bool) -> bool:

@@ -79,6 +79,8 @@ class HipZerusun(Res32Decoder):
                          if l.mixer.kind == "latent_attention"}
             self.gate = z(T * max(m.heads for m in lat))
             self.olat = z(T * max(m.heads * m.kv_rank for m in lat), dtype=el)
+            # key-slice partials of the decode attention (csrc/attention_latent.hip): up to 1024 (token, 16 heads, slice) units
+            self.att_ws = z(1024 * (max(m.kv_rank for m in lat) * 16 + 32)) if any(self.mfma.values()) else None
         if lin:
             self.o = z(T * max(m.heads * m.vdim for m in lin))
         ffs = [2 * m.ff for m in dense] + [2 * m.top * m.ff for m in moes] + [2 * m.shared_ff for m in moes]
@@ -227,7 +229,7 @@ class HipZerusun(Res32Decoder):
                                 H.GR_ELEM if mf else H.GR_F32)
             H.latent_attn(self.q_lat if mf else self.q_abs, self.q, self.kv[run], self.gate, meta.block_tables, self.max_blocks, positions,
                           meta.B, T, Hh, D, R, Cr, self.block_size, m.window, m.scale, freqs, mag, m.rope.dims, self.olat, f,
-                          q_abs_elem=mf, **seqs)
+                          q_abs_elem=mf, workspace=self.att_ws, **seqs)
             H.gemm_rows_batched(self.olat, w[p + "uv"], self.att, T, m.vdim, Cr, Hh, Hh * Cr, Cr, Hh * m.vdim, m.vdim, f, H.GR_ELEM)
         else:
             Hh, D, Dv = m.heads, m.dim, m.vdim

@@ -394,7 +394,8 @@ int ssd_sandwich_tail(const void* y_rows, const void* ydn_rows, const int32_t* i
 int ssd_rows_f32_to_bf16(const void* src, void* dst, int rows, int cols, long ld_src, long ld_dst, void* stream);
 
 /* y = x w^T for row-major x [M][K] and w [N][K] of ANY sizes (csrc/gemm_rows.hip).  epilogue 0: fp32 rows; 1: relu(y)^2 as
- * element-type rows; 2: element-type rows. */
+ * element-type rows; 2: element-type rows; 3 / 4 (bf16 only, N even): w rows are (gate, up) pairs -- row 2i, row 2i + 1 -- and y is
+ * act(gate) * up as element-type rows [M][N / 2], act = silu (3) or tanh-form gelu (4). */
 int ssd_gemm_rows(const void* x_rows, const void* w_rows, void* y, int M, int N, int K, int epilogue, int f32, void* stream);
 /* The same product per group: sorted rows offsets[e] .. offsets[e+1]-1 (e < E) multiply by w_rows + e * N * K; row_idx (optional)
  * names the x row of sorted row r as row_idx[r] / idx_div, y rows are the sorted rows.  rows = offsets[E]'s upper bound. */

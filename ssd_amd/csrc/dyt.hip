@@ -7,7 +7,7 @@
 //                        (+ sigmoid(gate logit) * shared row), or nothing; then the next layer's dyt(x) as GEMM-input rows, or the
 //                        element-type copy of x into the left half of the [x | x0] rows
 //  * ssd_glu_rows        out = act(a) * b for fp32 rows [a | b] (gate and up projections stacked), act = silu or tanh-form gelu
-// Everything is elementwise in fp32; a row's result depends on that row alone.  `f32` selects the element type of weights and of
+// Everything is elementwise in fp32 (grid = rows x column blocks); a row's result depends on that row alone.  `f32` selects the element type of weights and of
 // GEMM-input rows: 0 = bf16, 1 = fp32.  alpha is read from device memory (a one-element tensor of the checkpoint, kept as fp32).
 #include "common.h"
 
@@ -32,7 +32,7 @@ dyt_embed_kernel(const int64_t* __restrict__ ids, const T* __restrict__ table, c
   const bool ok = id >= 0 && id < vocab;
   const T* src = table + (size_t)(ok ? id : 0) * W;
   const float a = *alpha;
-  for (int c = threadIdx.x; c < W; c += 256) {
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < W; c += 256 * gridDim.y) {
     const float e = ok ? ldf<T>(src + c) : 0.f;
     const float v = tanhf(a * e) * ldf<T>(w + c) + ldf<T>(b + c);
     x[(size_t)t * W + c] = v;
@@ -49,7 +49,7 @@ dyt_rows_kernel(float* __restrict__ x, const T* __restrict__ add_vec, const floa
   const int ri = gather ? gather[ro] : ro;
   float* xr = x + (size_t)ri * W;
   const float a = *alpha;
-  for (int c = threadIdx.x; c < W; c += 256) {
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < W; c += 256 * gridDim.y) {
     float v = xr[c];
     if (add_vec) { v += ldf<T>(add_vec + c); xr[c] = v; }
     stf<T>(out + (size_t)ro * W + c, tanhf(a * v) * ldf<T>(w + c) + ldf<T>(b + c));
@@ -67,7 +67,7 @@ parallel_tail_kernel(float* __restrict__ x, const float* __restrict__ y_mix, con
   float* xr = x + (size_t)t * W;
   const float sg = (shared && sgate) ? sigmoidf_(sgate[(size_t)t * ld_sgate]) : 1.0f;
   const float a = next_out ? *alpha : 0.f;
-  for (int c = threadIdx.x; c < W; c += 256) {
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < W; c += 256 * gridDim.y) {
     float ff = 0.f;
     if (y_ff) {
       ff = y_ff[(size_t)t * W + c];
@@ -87,7 +87,7 @@ __global__ void __launch_bounds__(256)
 glu_rows_kernel(const float* __restrict__ ab, T* __restrict__ out, int F, int act) {
   const size_t r = blockIdx.x;
   const float* a = ab + r * 2 * F;
-  for (int c = threadIdx.x; c < F; c += 256) {
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < F; c += 256 * gridDim.y) {
     const float z = a[c], u = a[F + c];
     float g;
     if (act == 0) g = z * sigmoidf_(z);
@@ -100,15 +100,23 @@ glu_rows_kernel(const float* __restrict__ ab, T* __restrict__ out, int F, int ac
 
 #define LAUNCH_OK() (hipGetLastError() == hipSuccess ? SSD_OK : SSD_ERR_LAUNCH)
 
+// rows x column blocks: everything here is elementwise, so a few rows (decoding) still spread over the chip
+static inline dim3 row_grid(int rows, int cols) {
+  int cb = (cols + 255) / 256;
+  if (rows >= 1024) cb = 1;
+  else if (cb > 64) cb = 64;
+  return dim3(rows, cb);
+}
+
 extern "C" int ssd_dyt_embed(const int64_t* ids, const void* table, const float* alpha, const void* weight, const void* bias, void* x,
                              void* x0, void* cat, long ld_cat, int T, int W, long vocab, int f32, void* stream) {
   if (!ids || !table || !alpha || !weight || !bias || !x) return SSD_ERR_ARG;
   if (T <= 0 || W <= 0 || vocab <= 0 || (cat && ld_cat < W)) return SSD_ERR_SHAPE;
   if (f32)
-    hipLaunchKernelGGL(dyt_embed_kernel<float>, dim3(T), dim3(256), 0, (hipStream_t)stream, ids, (const float*)table, alpha,
+    hipLaunchKernelGGL(dyt_embed_kernel<float>, row_grid(T, W), dim3(256), 0, (hipStream_t)stream, ids, (const float*)table, alpha,
                        (const float*)weight, (const float*)bias, (float*)x, (float*)x0, (float*)cat, ld_cat, W, vocab);
   else
-    hipLaunchKernelGGL(dyt_embed_kernel<bf16_t>, dim3(T), dim3(256), 0, (hipStream_t)stream, ids, (const bf16_t*)table, alpha,
+    hipLaunchKernelGGL(dyt_embed_kernel<bf16_t>, row_grid(T, W), dim3(256), 0, (hipStream_t)stream, ids, (const bf16_t*)table, alpha,
                        (const bf16_t*)weight, (const bf16_t*)bias, (float*)x, (float*)x0, (bf16_t*)cat, ld_cat, W, vocab);
   return LAUNCH_OK();
 }
@@ -118,10 +126,10 @@ extern "C" int ssd_dyt_rows(void* x, const void* add_vec, const float* alpha, co
   if (!x || !alpha || !weight || !bias || !out_rows) return SSD_ERR_ARG;
   if (T <= 0 || W <= 0 || (gather && add_vec)) return SSD_ERR_SHAPE;
   if (f32)
-    hipLaunchKernelGGL(dyt_rows_kernel<float>, dim3(T), dim3(256), 0, (hipStream_t)stream, (float*)x, (const float*)add_vec, alpha,
+    hipLaunchKernelGGL(dyt_rows_kernel<float>, row_grid(T, W), dim3(256), 0, (hipStream_t)stream, (float*)x, (const float*)add_vec, alpha,
                        (const float*)weight, (const float*)bias, (float*)out_rows, gather, W);
   else
-    hipLaunchKernelGGL(dyt_rows_kernel<bf16_t>, dim3(T), dim3(256), 0, (hipStream_t)stream, (float*)x, (const bf16_t*)add_vec, alpha,
+    hipLaunchKernelGGL(dyt_rows_kernel<bf16_t>, row_grid(T, W), dim3(256), 0, (hipStream_t)stream, (float*)x, (const bf16_t*)add_vec, alpha,
                        (const bf16_t*)weight, (const bf16_t*)bias, (bf16_t*)out_rows, gather, W);
   return LAUNCH_OK();
 }
@@ -135,12 +143,12 @@ extern "C" int ssd_parallel_tail(void* x, const void* y_mix, const void* y_ff, c
   if (next_out && (!next_alpha || !next_weight || !next_bias)) return SSD_ERR_ARG;
   if (T <= 0 || W <= 0 || (ydn_rows && !y_ff && top <= 0) || (cat && ld_cat < W)) return SSD_ERR_SHAPE;
   if (f32)
-    hipLaunchKernelGGL(parallel_tail_kernel<float>, dim3(T), dim3(256), 0, (hipStream_t)stream, (float*)x, (const float*)y_mix,
+    hipLaunchKernelGGL(parallel_tail_kernel<float>, row_grid(T, W), dim3(256), 0, (hipStream_t)stream, (float*)x, (const float*)y_mix,
                        (const float*)y_ff, (const float*)ydn_rows, inv, weights, top, (const float*)shared_rows, shared_gate,
                        ld_shared_gate, next_alpha, (const float*)next_weight, (const float*)next_bias, (float*)next_out, (float*)cat,
                        ld_cat, W);
   else
-    hipLaunchKernelGGL(parallel_tail_kernel<bf16_t>, dim3(T), dim3(256), 0, (hipStream_t)stream, (float*)x, (const float*)y_mix,
+    hipLaunchKernelGGL(parallel_tail_kernel<bf16_t>, row_grid(T, W), dim3(256), 0, (hipStream_t)stream, (float*)x, (const float*)y_mix,
                        (const float*)y_ff, (const float*)ydn_rows, inv, weights, top, (const float*)shared_rows, shared_gate,
                        ld_shared_gate, next_alpha, (const bf16_t*)next_weight, (const bf16_t*)next_bias, (bf16_t*)next_out,
                        (bf16_t*)cat, ld_cat, W);
@@ -151,10 +159,10 @@ extern "C" int ssd_glu_rows(const void* ab_rows, void* out_rows, int rows, int F
   if (!ab_rows || !out_rows) return SSD_ERR_ARG;
   if (rows <= 0 || F <= 0 || act < 0 || act > 1) return SSD_ERR_SHAPE;
   if (f32)
-    hipLaunchKernelGGL(glu_rows_kernel<float>, dim3(rows), dim3(256), 0, (hipStream_t)stream, (const float*)ab_rows, (float*)out_rows,
+    hipLaunchKernelGGL(glu_rows_kernel<float>, row_grid(rows, F), dim3(256), 0, (hipStream_t)stream, (const float*)ab_rows, (float*)out_rows,
                        F, act);
   else
-    hipLaunchKernelGGL(glu_rows_kernel<bf16_t>, dim3(rows), dim3(256), 0, (hipStream_t)stream, (const float*)ab_rows,
+    hipLaunchKernelGGL(glu_rows_kernel<bf16_t>, row_grid(rows, F), dim3(256), 0, (hipStream_t)stream, (const float*)ab_rows,
                        (bf16_t*)out_rows, F, act);
   return LAUNCH_OK();
 }

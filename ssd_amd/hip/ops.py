@@ -406,7 +406,7 @@ def rows_f32_to_bf16(src, dst, rows: int, cols: int, ld_src: int, ld_dst: int):
     _check(load_library().ssd_rows_f32_to_bf16(_p(src), _p(dst), rows, cols, ld_src, ld_dst, _stream()), "ssd_rows_f32_to_bf16")
 
 
-GR_F32, GR_RELU2, GR_ELEM = 0, 1, 2
+GR_F32, GR_RELU2, GR_ELEM, GR_GLU_SILU, GR_GLU_GELU = 0, 1, 2, 3, 4
 
 
 def gemm_rows(x, w, y, M: int, N: int, K: int, f32: bool, epilogue: int = GR_F32):

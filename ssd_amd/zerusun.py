@@ -8,9 +8,9 @@ Launches per layer run (T token rows):
     latent attention   [dq | dkv | gate] GEMM -> latent_store (norms, rope, cache row, gates) -> W_uq GEMM -> per-head W_uk^T GEMM
                        (queries into the latent space) -> latent_attn -> per-head W_uv GEMM -> W_o GEMM
     linear attention   [q | k | v | g] GEMM -> lightning_scan (state slot) -> lightning_gate_norm -> W_o GEMM
-    dense ff           [gate | up] GEMM -> glu_rows -> down GEMM
-    routed ff          [router | shared gate] GEMM -> moe_route_softmax -> moe_plan -> grouped [gate | up] GEMM -> glu_rows -> grouped
-                       down GEMM -> shared [gate | up] GEMM -> glu_rows -> shared down GEMM
+    dense ff           [gate | up] GEMM with the GLU as epilogue (fp32 mode: + glu_rows) -> down GEMM
+    routed ff          [router | shared gate] GEMM -> moe_route_softmax -> moe_plan -> grouped [gate | up] GEMM (GLU epilogue) ->
+                       grouped down GEMM -> shared [gate | up] GEMM (GLU epilogue) -> shared down GEMM
     parallel_tail      x += mixer + ff (the routed mix rides along) and the next layer's norm, or the [x | x0] row of a loop entry
 over pre-allocated buffers (nothing is allocated during a forward).  Same interface as ssd_amd.model.HipDecoder towards the ModelRunner.
 
@@ -85,7 +85,7 @@ class HipZerusun(Res32Decoder):
             self.o = z(T * max(m.heads * m.vdim for m in lin))
         ffs = [2 * m.ff for m in dense] + [2 * m.top * m.ff for m in moes] + [2 * m.shared_ff for m in moes]
         if ffs:
-            self.ab = z(T * max(ffs))                                        # fp32 [gate | up] rows
+            self.ab = z(T * max(ffs)) if self.f32 else None                   # fp32 [gate | up] rows (bf16: the GEMM epilogue applies the GLU)
             self.act = z(T * max(ffs) // 2, dtype=el)
         if moes:
             top = max(m.top for m in moes)
@@ -122,8 +122,12 @@ class HipZerusun(Res32Decoder):
             w[n], w[n + ".b"] = cv(raw[n]), cv(raw[n + ".b"])
             w[n + ".alpha"] = raw[n + ".alpha"].float().reshape(1).contiguous()
 
+        def pair(gate, up):
+            # bf16: rows interleaved (gate_0, up_0, gate_1, ...) for the GEMM's paired epilogue; fp32: [gate | up], a GLU launch follows
+            return torch.stack([gate, up], dim=1).reshape(-1, gate.shape[1]) if not self.f32 else torch.cat([gate, up], dim=0)
+
         def glu(dst, src):
-            w[dst + "gu"] = cv(torch.cat([raw[src + "gate"], raw[src + "up"]], dim=0))
+            w[dst + "gu"] = cv(pair(raw[src + "gate"], raw[src + "up"]))
             w[dst + "down"] = cv(raw[src + "down"])
 
         w["embed"] = cv(raw["embed"])
@@ -150,8 +154,7 @@ class HipZerusun(Res32Decoder):
             if ml.kind == "dense":
                 glu(p + "mlp.", p + "mlp.")
                 continue
-            w[p + "mlp.gu"] = cv(torch.stack([torch.cat([raw[p + f"mlp.e{e}.gate"], raw[p + f"mlp.e{e}.up"]], dim=0)
-                                              for e in range(ml.experts)]))
+            w[p + "mlp.gu"] = cv(torch.stack([pair(raw[p + f"mlp.e{e}.gate"], raw[p + f"mlp.e{e}.up"]) for e in range(ml.experts)]))
             w[p + "mlp.down"] = cv(torch.stack([raw[p + f"mlp.e{e}.down"] for e in range(ml.experts)]))
             if ml.shared_ff:
                 w[p + "mlp.router"] = cv(torch.cat([raw[p + "mlp.router"], raw[p + "mlp.shared.sg"].reshape(1, -1)], dim=0))
@@ -246,8 +249,7 @@ class HipZerusun(Res32Decoder):
         if ml is None:
             return {}
         if ml.kind == "dense":
-            H.gemm_rows(self.hn, w[p + "gu"], self.ab, T, 2 * ml.ff, W, f)
-            H.glu_rows(self.ab, self.act, T, ml.ff, H.GLU_GELU_TANH, f)
+            self._glu_gemm(self.hn, w[p + "gu"], T, ml.ff, H.GLU_GELU_TANH)
             H.gemm_rows(self.act, w[p + "down"], self.y_ff, T, W, ml.ff, f)
             return dict(y_ff=self.y_ff)
         E, top = ml.experts, ml.top
@@ -255,17 +257,29 @@ class HipZerusun(Res32Decoder):
         H.gemm_rows(self.hn, w[p + "router"], self.r_z, T, ldz, W, f)
         H.moe_route_softmax(self.r_z, ldz, self.r_idx, self.r_wt, T, E, top, ml.groups, ml.keep, ml.scale)
         H.moe_plan(self.r_idx, T, top, E, self.r_off, self.r_perm, self.r_inv)
-        H.gemm_rows_grouped(self.hn, w[p + "gu"], self.ab, self.r_off, E, T * top, 2 * ml.ff, W, f, H.GR_F32, row_idx=self.r_perm,
-                            idx_div=top)
-        H.glu_rows(self.ab, self.act, T * top, ml.ff, H.GLU_SILU, f)
+        if f:
+            H.gemm_rows_grouped(self.hn, w[p + "gu"], self.ab, self.r_off, E, T * top, 2 * ml.ff, W, f, H.GR_F32, row_idx=self.r_perm,
+                                idx_div=top)
+            H.glu_rows(self.ab, self.act, T * top, ml.ff, H.GLU_SILU, f)
+        else:
+            H.gemm_rows_grouped(self.hn, w[p + "gu"], self.act, self.r_off, E, T * top, 2 * ml.ff, W, f, H.GR_GLU_SILU, row_idx=self.r_perm,
+                                idx_div=top)
         H.gemm_rows_grouped(self.act, w[p + "down"], self.ydn, self.r_off, E, T * top, W, ml.ff, f, H.GR_F32)
         out = dict(ydn=self.ydn, inv=self.r_inv, weights=self.r_wt, top=top)
         if ml.shared_ff:
-            H.gemm_rows(self.hn, w[p + "shared.gu"], self.ab, T, 2 * ml.shared_ff, W, f)
-            H.glu_rows(self.ab, self.act, T, ml.shared_ff, H.GLU_SILU, f)
+            self._glu_gemm(self.hn, w[p + "shared.gu"], T, ml.shared_ff, H.GLU_SILU)
             H.gemm_rows(self.act, w[p + "shared.down"], self.ysh, T, W, ml.shared_ff, f)
             out.update(shared=self.ysh, shared_gate=self.r_z.view(-1)[E:], ld_shared_gate=ldz)
         return out
+
+    def _glu_gemm(self, x, w_gu, T: int, ff: int, act: int) -> None:
+        """self.act = act(W_gate x) * (W_up x): in bf16 the GEMM's paired epilogue (weight rows interleaved at load), in fp32 a
+        [gate | up] GEMM with fp32 rows out and the GLU launch."""
+        if self.f32:
+            H.gemm_rows(x, w_gu, self.ab, T, 2 * ff, self.W, True)
+            H.glu_rows(self.ab, self.act, T, ff, act, True)
+        else:
+            H.gemm_rows(x, w_gu, self.act, T, 2 * ff, self.W, False, H.GR_GLU_SILU if act == H.GLU_SILU else H.GR_GLU_GELU)
 
     def _enters_pass(self, run: int) -> bool:
         return self.cfg.has_loop and self.runs[run][0] == self.cfg.loop_start

@@ -91,6 +91,30 @@ def test_glu_rows_and_batched_gemm(f32):
         assert torch.allclose(y[:, :G * N].cpu().double(), ref, **tol(f32)) and bool((y[:, G * N:] == 7.0).all())
 
 
+@pytest.mark.parametrize("M", [1, 9, 200])
+def test_gemm_with_the_glu_as_epilogue(M):
+    """bf16: weight rows in (gate, up) pairs, output act(gate) * up -- the tile form, the skinny form, dense and per expert."""
+    K, F, E = 72, 44, 3
+    x = rnd(M, K, seed=1).bfloat16()
+    gate, up = rnd(E, F, K, seed=2, scale=0.3).bfloat16(), rnd(E, F, K, seed=3, scale=0.3).bfloat16()
+    pairs = torch.stack([gate, up], dim=2).reshape(E, 2 * F, K).contiguous()
+    for epi, fn in ((H().GR_GLU_SILU, Z.silu), (H().GR_GLU_GELU, Z.gelu_tanh)):
+        y = torch.zeros(M, F, dtype=torch.bfloat16, device=DEV)
+        H().gemm_rows(x.to(DEV), pairs[0].contiguous().to(DEV), y, M, 2 * F, K, False, epi)
+        ref = fn(x.double() @ gate[0].double().T) * (x.double() @ up[0].double().T)
+        assert torch.allclose(y.cpu().double(), ref, rtol=2e-2, atol=2e-2)
+    # grouped: rows sorted by expert
+    cnt = [M // 3, 0, M - M // 3]
+    off = torch.tensor([0, cnt[0], cnt[0], M], dtype=torch.int32)
+    y = torch.zeros(M, F, dtype=torch.bfloat16, device=DEV)
+    H().gemm_rows_grouped(x.to(DEV), pairs.to(DEV), y, off.to(DEV), E, M, 2 * F, K, False, H().GR_GLU_SILU)
+    which = torch.tensor([0] * cnt[0] + [2] * cnt[2])
+    ref = torch.stack([Z.silu(x[r].double() @ gate[which[r]].double().T) * (x[r].double() @ up[which[r]].double().T) for r in range(M)])
+    assert torch.allclose(y.cpu().double(), ref, rtol=2e-2, atol=2e-2)
+    with pytest.raises(Exception):
+        H().gemm_rows(x.float().to(DEV), pairs[0].float().contiguous().to(DEV), y, M, 2 * F, K, True, H().GR_GLU_SILU)
+
+
 @pytest.mark.parametrize("E,top,groups,keep", [(16, 4, 2, 1), (12, 3, 3, 2), (8, 2, 1, 1), (6, 6, 3, 3), (5, 1, 5, 1), (130, 8, 10, 3)])
 def test_softmax_router_with_group_limited_choice(E, top, groups, keep):
     T, ld = 33, E + 1

@@ -190,3 +190,20 @@ def test_scheduler_and_trace_engine_hand_out_state_slots(tmp_path):
     assert prefill and picked == [seqs[1]] and seqs[1].state_slot == 1
     with pytest.raises(AssertionError):
         Config(str(tmp_path), speculate=True, draft=str(tmp_path), speculate_k=2, kvcache_block_size=16)
+
+
+def test_bench_option_and_equal_size_pairs():
+    """bench.py accepts --workload zerusun next to its default; every benchmarked size pairs a Zerusun model with a Fatulix model of the
+    same width, layers, vocabulary, experts, top and feed-forward parameters per token."""
+    import bench
+    from ssd_amd.utils import arch_bench
+    assert bench.parse([]).workload == "c4"                                  # the default workload is untouched
+    a = bench.parse(["--workload", "zerusun", "--arch-size", "w2048", "--arch-batch", "1", "--arch-only", "zerusun"])
+    assert a.workload == "zerusun" and a.arch_size == "w2048" and a.arch_batch == 1 and a.arch_only == "zerusun"
+    for size in arch_bench.SIZES:
+        zer, fat = arch_bench.zerusun_models(size)
+        assert zer.hidden_size == fat.hidden_size and zer.vocab_size == fat.vocab_size and len(zer.runs()) == len(fat.runs())
+        assert {l.mixer.kind for l in zer.layers} == {"latent_attention", "lightning"} and zer.recurrent
+        mz, mf = zer.layers[0].mlp, fat.layers[0].mlp
+        assert (mz.experts, mz.top) == (mf.experts, mf.top)
+        assert 3 * (mz.top * mz.ff + mz.shared_ff) == 2 * (mf.top * mf.ff + mf.shared_ff)

@@ -143,11 +143,13 @@ def _pages(n_seq, lens, bs, seed):
 @pytest.mark.parametrize("Hh,D,R,Cr,Qr,win,rd,bs", [(6, 32, 32, 128, 64, 40, 32, 64), (3, 8, 6, 20, 12, 5, 4, 16), (5, 16, 8, 72, 40, 0, 8, 16),
                                                     (1, 8, 2, 8, 8, 1, 2, 16), (20, 16, 64, 512, 32, 33, 48, 16), (17, 8, 32, 32, 16, 0, 32, 32),
                                                     (16, 8, 32, 288, 16, 32, 2, 16)])
-def test_latent_store_and_windowed_attention_over_scattered_pages(f32, Hh, D, R, Cr, Qr, win, rd, bs):
+@pytest.mark.parametrize("lens", [[37, 50], [333, 207]])
+def test_latent_store_and_windowed_attention_over_scattered_pages(f32, Hh, D, R, Cr, Qr, win, rd, bs, lens):
     """Two sequences; the second arrives in two launches (a portion, then the rest) and must see the keys of the first launch.  Where the
     MFMA form takes the sizes (bf16, latent sizes in multiples of 32) it is the one that runs, with the latent-space queries as bf16 rows."""
     el = elem(f32)
-    lens = [37, 50]
+    if lens[0] > 100:
+        win = win * 5          # windows of many key steps, ending inside and at the borders of pages
     eps, scale = 1e-5, 0.2
     freqs, mag = Z.rope_frequencies(rd, 10000.0, {"factor": 4.0, "original": 32, "fast": 16.0, "slow": 1.0})
     NP = Qr + Cr + R + Hh
@@ -183,9 +185,12 @@ def test_latent_store_and_windowed_attention_over_scattered_pages(f32, Hh, D, R,
                         f32, cu_q=d(cu), q_abs_elem=mfma, workspace=ws)
         return cq, out
 
-    cq1, o1 = launch([(0, 0, 37), (1, 0, 21)])
-    cq2, o2 = launch([(1, 21, 50)])
-    got = {0: o1[:37], 1: torch.cat([o1[37:], o2])}
+    n0, n1 = lens
+    cut = n1 * 2 // 5 + 1
+    cq1, o1 = launch([(0, 0, n0), (1, 0, cut)])
+    cq2, o2 = launch([(1, cut, n1 - 3)])
+    o3 = [launch([(1, t, t + 1)])[1] for t in range(n1 - 3, n1)]             # single rows: the key-slice form where it applies
+    got = {0: o1[:n0], 1: torch.cat([o1[n0:], o2] + o3)}
     for s, n in enumerate(lens):
         pr = proj_all[s].double()
         c = Z.rms(pr[:, Qr:Qr + Cr], wkv.double(), eps)
@@ -201,7 +206,7 @@ def test_latent_store_and_windowed_attention_over_scattered_pages(f32, Hh, D, R,
         ref = torch.einsum("hij,jc->ihc", p, c) * torch.sigmoid(pr[:, Qr + Cr + R:])[..., None]
         assert torch.allclose(got[s].cpu().double().view(n, Hh, Cr), ref, **tol(f32)), s
     ref_cq = Z.rms(proj_all[0][:, :Qr].double(), wq.double(), eps)
-    assert torch.allclose(cq1[:37].cpu().double(), ref_cq, **tol(f32))
+    assert torch.allclose(cq1[:n0].cpu().double(), ref_cq, **tol(f32))
 
 
 @pytest.mark.parametrize("Hh,D,Dv", [(6, 32, 32), (3, 16, 24), (1, 8, 1), (2, 40, 130), (2, 128, 128), (3, 64, 96), (1, 256, 32), (2, 32, 48)])

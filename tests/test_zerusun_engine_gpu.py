@@ -62,6 +62,18 @@ def configs():
                                               mlp=M(experts=3, top=3, groups=None, ff=20, shared_ff=12)),
                                             S(heads=5, dim=12, vdim=20, mlp=D(52)), L(window=0, scaling=None)],
                                            vocab=77, width=50, loop=(0, 0, 1)),
+        # sizes the bf16 fast forms take: latent sizes in multiples of 32 (MFMA attention; 20 heads = two head tiles, one partly empty),
+        # state sizes of the register scan; windows of several 32-key steps
+        "fast_forms": Z.make_config([S(heads=2, dim=32, vdim=64, mlp=D(48)),
+                                     L(heads=20, dim=16, rot_dim=32, vdim=8, q_rank=48, kv_rank=64, window=70, mlp=M(experts=4, groups=(2, 2))),
+                                     L(heads=3, dim=8, rot_dim=32, vdim=16, q_rank=16, kv_rank=32, window=0, rot_dims=8, scaling=None),
+                                     S(heads=3, dim=64, vdim=32, mlp=M(experts=4, top=1, groups=None, shared_ff=0))],
+                                    vocab=120, width=96, loop=(1, 3, 2)),
+        # one kind of mixer only: no cache pages at all (every layer keeps a state) / no state slots at all
+        "only_linear": Z.make_config([S(mlp=D()), S(heads=2, dim=24, vdim=8, mlp=M(experts=2, top=1, groups=(2, 2), shared_ff=0))], vocab=40,
+                                     width=48, loop=(0, 1, 2)),
+        "only_latent": Z.make_config([L(window=6, mlp=M(experts=4, groups=(4, 2))), L(heads=2, window=0, mlp=None)], vocab=40, width=48,
+                                     loop=(1, 2, 2)),
         # the loop is the tail of the stack, two passes; recurrent layers only inside it
         "loop_tail": Z.make_config([L(window=17, mlp=D()), S(mlp=D(24)), S(heads=4, dim=32, vdim=16, mlp=M())], vocab=64, width=64,
                                    loop=(1, 3, 2)),
@@ -205,6 +217,39 @@ def test_mixed_batches_of_unequal_requests_with_pages_and_slots_used_again(tmp_p
         for r in ("a", "e"):
             alone = _replay(eng, r + "x", reqs[r], [len(reqs[r])])
             assert torch.equal(alone, torch.cat(got[r]))
+
+
+@pytest.mark.parametrize("block_size", [32, 64])
+def test_bf16_fast_forms_through_the_engine_portions_decoding_and_mixed_steps(tmp_path, block_size):
+    """bf16 with 32 / 64-token pages and sizes that the MFMA attention and the register scan take: whole prompt, portions cut at and next
+    to page borders, decoded tokens (the key-slice form of the attention), two requests sharing steps; every position against the oracle,
+    and the portions against the whole prompt (the same bf16 inputs, other fp32 summation orders only)."""
+    cfg, w = make("fast_forms", seed=9)
+    n = 190
+    ta, tb = tokens(n, cfg["vocab"], 30), tokens(77, cfg["vocab"], 31)
+    ra, rb = Z.forward(cfg, w, ta), Z.forward(cfg, w, tb)
+    eng = engine(tmp_path, cfg, w, "bfloat16", max_tokens=384, block_size=block_size)
+    m = eng.runner.model
+    assert all(m.mfma.values()) and m.att_ws is not None
+    whole = _replay(eng, "w", ta, [n])
+    assert close(whole, ra, "bfloat16"), rel_err(whole, ra)
+    cuts = sorted({block_size - 1, block_size, block_size + 1, 2 * block_size + 2, 150} | set(range(151, n + 1)))
+    got = _replay(eng, "c", ta, cuts)
+    assert close(got, ra, "bfloat16"), rel_err(got, ra)
+    assert row_err(got, whole.double().cpu()).median() < 0.02
+    ga, gb, ia, ib = [], [], 0, 0
+    for ka, kb in [(40, 1), (1, 1), (1, 30), (25, 1), (1, 44)] + [(1, 0)] * 10 + [(n - 78, 0)]:
+        entries = []
+        if ka:
+            entries.append({"id": "a", "tokens": ta[ia:ia + ka], "want": list(range(ka))})
+        if kb:
+            entries.append({"id": "b", "tokens": tb[ib:ib + kb], "want": list(range(kb))})
+        ia, ib = ia + ka, ib + kb
+        out = eng.step(entries, [r for r, done in (("a", ia == n), ("b", ib == 77 and kb)) if done])
+        ga.append(out[:ka])
+        gb.append(out[ka:ka + kb])
+    assert ia == n and ib == 77
+    assert close(torch.cat(ga), ra, "bfloat16") and close(torch.cat(gb), rb, "bfloat16")
 
 
 def test_long_decoding_over_many_pages(tmp_path):
